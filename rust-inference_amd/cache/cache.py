@@ -31,10 +31,15 @@ PAGE_SIZE = 32   # tokens per page, as in the reference (src/kvcache.rs:12)
 @dataclass(frozen=True)
 class KVNeed:
     """Keys and values of ``kv_heads`` heads of ``head_dim`` for every token, or for
-    the last ``window`` tokens only."""
+    the last ``window`` tokens only.  ``v_dim``: the size of a value head where it is not ``head_dim``."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_dim: Optional[int] = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.v_dim or self.head_dim
 
 
 @dataclass(frozen=True)
@@ -49,7 +54,7 @@ class KVGroup:
 
     ``k_pages[e]`` is ``[num_pages, kv_heads, page_size, head_dim]`` for entry ``e`` of
     the group (the reference's layout: src/kvcache.rs:42-50, :145-147).  ``v_pages[e]`` is
-    ``[num_pages, kv_heads, head_dim, page_size]``: values lie transposed inside a page,
+    ``[num_pages, kv_heads, v_dim, page_size]``: values lie transposed inside a page,
     the page's tokens contiguous for each channel, because that is the operand order
     the matrix cores want for the product of weights and values.  One page number
     means the same page in every entry.
@@ -61,7 +66,7 @@ class KVGroup:
         self.pool = PagePool(num_pages, page_size, num_slots, max_pages_per_slot, need.window)
         self.index_of = {e: i for i, e in enumerate(self.entries)}
         k_shape = (len(self.entries), num_pages, need.kv_heads, page_size, need.head_dim)
-        v_shape = (len(self.entries), num_pages, need.kv_heads, need.head_dim, page_size)
+        v_shape = (len(self.entries), num_pages, need.kv_heads, need.value_dim, page_size)
         self.k_pages = torch.zeros(k_shape, dtype=dtype, device=device) if allocate else None
         self.v_pages = torch.zeros(v_shape, dtype=dtype, device=device) if allocate else None
 

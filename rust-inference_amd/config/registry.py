@@ -3,7 +3,8 @@
 An entry holds the configuration class that reads the architecture's config.json
 and the function that turns that configuration into a ``ModelSpec`` (the list of
 layers, their parts and the order they run in).  The reference dispatches on
-``architectures[0]`` and falls back to ``model_type`` (src/models/config.rs:139-145).
+``architectures[0]`` and falls back to ``model_type`` (src/models/config.rs:139-145); a config.json that names
+its design in a single ``architecture`` string is resolved by that.
 """
 from __future__ import annotations
 
@@ -43,6 +44,10 @@ def resolve_architecture(raw: dict) -> Architecture:
     """The registry entry a config.json selects, by ``architectures[0]`` and else by
     ``model_type``; an unknown name is an error that lists the known ones."""
     archs = raw.get("architectures") or []
+    if not archs and isinstance(raw.get("architecture"), str):
+        archs = [raw["architecture"]]
+    elif isinstance(raw.get("architecture"), str) and raw["architecture"] in _BY_NAME:
+        archs = [raw["architecture"]]
     name = archs[0] if archs else None
     if name is None:
         name = _ALIASES.get(raw.get("model_type"))

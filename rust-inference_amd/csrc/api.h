@@ -49,11 +49,60 @@ int ri_qk_norm_rope_kv_write(void* qkv, int act_dtype, const float* q_gain, cons
 
 // Causal grouped-query attention of each new token over its sequence's pages (any number of new tokens
 // per sequence).  q is read from qkv rows (row stride q_stride elements); out: [tokens, heads * head_dim].
-// window <= 0: all keys 0..pos; else keys max(0, pos - window + 1)..pos.
+// window <= 0: all keys 0..pos; else keys max(0, pos - window + 1)..pos.  v_dim: the size of a value head
+// (v_pages: [pages, kv_heads, v_dim, page_size]; out: [tokens, heads * v_dim]).  softcap > 0: a score s becomes
+// softcap * tanh(s / softcap) before the softmax.
 int ri_attention(void* out, const void* q, int act_dtype, int q_stride, const void* k_pages, const void* v_pages,
                  int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table,
-                 int table_width, int tokens, int heads, int kv_heads, int head_dim, int page_size, int window,
-                 float scale, void* stream);
+                 int table_width, int tokens, int heads, int kv_heads, int head_dim, int v_dim, int page_size,
+                 int window, float scale, float softcap, void* stream);
+
+// Queries and keys for an attention without rotation, keys and values into their pages, from the fused
+// projection qkv: [tokens, heads * dim + kv_heads * dim + kv_heads * vdim].  Per-head RMS norm of q and k (gains
+// may be NULL), then q *= 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1) in place (temp_coef 0: none).
+// k_pages: [pages, kv_heads, page_size, dim]; v_pages: [pages, kv_heads, vdim, page_size].
+int ri_qk_norm_temper_kv_write(void* qkv, int act_dtype, const float* q_gain, const float* k_gain, float eps,
+                               float temp_coef, int temp_every, const int32_t* tok_pos, const int32_t* tok_seq,
+                               const int32_t* page_table, int table_width, void* k_pages, void* v_pages,
+                               int cache_dtype, int tokens, int heads, int kv_heads, int dim, int vdim, int page_size,
+                               void* stream);
+
+// Several residual streams per token (streams: [total_rows, n_streams, dim] float32), the write that waits for
+// them, the read and the norm, in one kernel.  For row r (rows == NULL: every row, and the new streams are stored;
+// else row rows[r], nothing stored):
+//   pending != NULL:  y = sum of its parts [parts, total_rows, dim];  x_t <- sum_s mix[s * n + t] x_s + out_coef[t] y
+//   u = sum_t in_coef[t] x_t;  out[r] = norm(u): norm_kind 0 none, 1 RMS (gain), 2 layer norm (gain, bias or NULL).
+// mix, out_coef, in_coef NULL: the identity, ones, ones (n_streams 1: residual += pending, then the norm).
+// fresh != NULL: [total_rows, dim], the one row every stream starts from; the call spreads it into `streams`.
+int ri_streams_read_norm(void* out, int out_dtype, float* streams, const float* fresh, int n_streams,
+                         const void* pending, int pending_dtype, int parts, int total_rows, const float* mix,
+                         const float* out_coef, const float* in_coef, const float* gain, const float* bias, float eps,
+                         int norm_kind, const int32_t* rows, int n_rows, int dim, void* stream);
+
+// out[t, :] = norm(table[ids[t], :] + positions[tok_pos[t], :]) as float32 (positions may be NULL; norm kinds as
+// above).  Both tables of table_dtype.
+int ri_embed_positions_norm(float* out, const void* table, const void* positions, int table_dtype, const int32_t* ids,
+                            const int32_t* tok_pos, const float* gain, const float* bias, float eps, int norm_kind,
+                            int tokens, int dim, void* stream);
+
+// Gated linear attention.  proj: [tokens, row] of act_dtype with, for each of `heads` heads, q and k of `dim`
+// and v of `vdim` at the column offsets q_off, k_off, v_off (head h at off + h * size); z: float32
+// [tokens, heads * dim], the decay's pre-activation without its bias (z_bias: [heads * dim] or NULL).  Per head,
+// with alpha = exp(log_sigmoid(z + bias) / tau):   S <- diag(alpha_t) S + k_t v_t^T,   o_t = S^T (q_t * q_scale).
+// state: float32 [slots, heads, dim, vdim], read at the sequence's slot before its first token of the step and
+// written back after its last.  cu_seqlens: [seqs + 1] over the flat tokens; slots: [seqs].  out: float32
+// [tokens, heads * vdim].
+int ri_gla_scan(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off, const float* z,
+                const float* z_bias, float tau, float q_scale, float* state, const int32_t* cu_seqlens,
+                const int32_t* slots, int seqs, int heads, int dim, int vdim, void* stream);
+
+// out[t, h, :] = rms_norm(o[t, h, :]) * gain * silu(gate[t, h, :]): o float32 [tokens, heads * vdim]; gate read
+// from proj rows at column g_off; out of act_dtype [tokens, heads * vdim].
+int ri_gla_norm_gate(void* out, const float* o, const void* proj, int act_dtype, int row, int g_off, const float* gain,
+                     float eps, int tokens, int heads, int vdim, void* stream);
+
+// out[i] = max(y[i], 0)^2.
+int ri_relu_squared(void* out, const void* y, int dtype, long total, void* stream);
 
 // The same attention on the matrix cores, for bfloat16, pages of 32 tokens and head_dim 32, 64 or 128.
 // Prefill form: any number of new tokens per sequence (cu_seqlens: int32 [seqs + 1] over the flat tokens,

@@ -1,0 +1,202 @@
+// Gated linear attention: a state of dim x vdim numbers per head and sequence instead of keys and values,
+//     S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,        o_t = S_t^T q_t,
+// with one decay per key channel, alpha = sigmoid(z)^(1/tau) = exp(log_sigmoid(z) / tau).  State, decay, its
+// logarithm and exponential, and the sums are float32; q, k, v and z come from products.
+//
+// The scan walks a sequence's tokens in order; what runs side by side is everything else: a workgroup owns one
+// (sequence, head) and GLA_COLS columns of the state, its 256 threads as 16 columns x 16 slices of rows, every
+// thread keeping its rows of its column in registers.  Tokens go through in blocks of nb: a block's q, k, alpha
+// and v are staged in LDS (two buffers), the next block's loads are asked for before the block in work is
+// computed and stored after it, so memory's latency is paid once a block and behind the arithmetic; the 16
+// slices' shares of o_t meet through a shuffle inside a wavefront and through LDS between the four wavefronts,
+// with one barrier a block.  The same kernel serves a step of one token.
+#include "api.h"
+#include "common.h"
+
+#define GLA_COLS 16
+#define GLA_SLICES 16
+#define GLA_MAX_ROWS 32          // rows of a column per thread: dim <= 16 * 32
+#define GLA_MAX_NB 8             // tokens of a block
+#define GLA_STAGE 4              // staged elements of q, k and z per thread and block: nb * dim <= 4 * 256
+
+__device__ __forceinline__ float log_sigmoid(float z) {
+    // min(z, 0) - log(1 + exp(-|z|)): no overflow on either side
+    return fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+}
+
+template <typename TA>
+__global__ void __launch_bounds__(256)
+gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, int q_off, int k_off, int v_off,
+                const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau, float q_scale,
+                float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
+                int heads, int dim, int vdim, int nb) {
+    extern __shared__ float lds[];                           // two buffers of nb tokens: q, k, alpha (dim each), v (16)
+    __shared__ float part[2][GLA_MAX_NB][4][GLA_COLS];       // the wavefronts' shares of o_t, two blocks in flight
+    const int b = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * GLA_COLS;
+    const int tid = threadIdx.x, c = tid % GLA_COLS, r = tid / GLA_COLS, wave = tid / RI_WAVE;
+    const int col = col0 + c;
+    const bool live = col < vdim;
+    const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
+    if (t1 <= t0) return;
+    const int stride = 3 * dim + GLA_COLS, per = nb * dim;
+    float* S = state + (((size_t)slots[b] * heads + h) * dim) * vdim + col;
+    float s[GLA_MAX_ROWS];
+#pragma unroll
+    for (int j = 0; j < GLA_MAX_ROWS; ++j) {
+        const int i = r + j * GLA_SLICES;
+        s[j] = (live && i < dim) ? S[(size_t)i * vdim] : 0.f;
+    }
+    const int rows_here = (dim - r + GLA_SLICES - 1) / GLA_SLICES;          // rows r, r + 16, ... below dim
+
+    // a block's inputs on their way: every load is issued whatever the indices are, from a token and a column
+    // pulled back inside the data
+    float rq[GLA_STAGE], rk[GLA_STAGE], rz[GLA_STAGE], rv;
+    auto ask = [&](int tb) {
+#pragma unroll
+        for (int j = 0; j < GLA_STAGE; ++j) {
+            const int e = min(tid + j * 256, per - 1);
+            const int tok = min(tb + e / dim, t1 - 1), i = e % dim;
+            const TA* x = proj + (size_t)tok * row;
+            rq[j] = to_f32(x[q_off + h * dim + i]);
+            rk[j] = to_f32(x[k_off + h * dim + i]);
+            rz[j] = z[((size_t)tok * heads + h) * dim + i];
+        }
+        const int e = min(tid, nb * GLA_COLS - 1);
+        const int tok = min(tb + e / GLA_COLS, t1 - 1), cc = min(col0 + e % GLA_COLS, vdim - 1);
+        rv = to_f32(proj[(size_t)tok * row + v_off + h * vdim + cc]);
+    };
+    auto put = [&](int which) {
+        float* buf = lds + (size_t)which * nb * stride;
+#pragma unroll
+        for (int j = 0; j < GLA_STAGE; ++j) {
+            const int e = tid + j * 256;
+            if (e < per) {
+                const int i = e % dim;
+                float* at = buf + (size_t)(e / dim) * stride;
+                at[i] = rq[j] * q_scale;
+                at[dim + i] = rk[j];
+                at[2 * dim + i] = expf(log_sigmoid(rz[j] + (z_bias ? z_bias[h * dim + i] : 0.f)) * inv_tau);
+            }
+        }
+        if (tid < nb * GLA_COLS) buf[(size_t)(tid / GLA_COLS) * stride + 3 * dim + tid % GLA_COLS] = rv;
+    };
+    ask(t0);
+    put(0);
+    __syncthreads();
+    int blk = 0;
+    for (int tb = t0; tb < t1; tb += nb, ++blk) {
+        ask(tb + nb);
+        const float* buf = lds + (size_t)(blk & 1) * nb * stride;
+        for (int n = 0; n < nb; ++n) {
+            if (tb + n >= t1) break;                         // the same for the whole workgroup
+            const float* at = buf + (size_t)n * stride;
+            const float v = at[3 * dim + c];
+            float o = 0.f;
+#pragma unroll
+            for (int j = 0; j < GLA_MAX_ROWS; ++j) {
+                if (j < rows_here) {
+                    const int i = r + j * GLA_SLICES;
+                    s[j] = at[2 * dim + i] * s[j] + at[dim + i] * v;
+                    o += s[j] * at[i];
+                }
+            }
+            // lanes of a wavefront: 4 slices x 16 columns
+            o += __shfl_xor(o, 16, RI_WAVE);
+            o += __shfl_xor(o, 32, RI_WAVE);
+            if ((tid & (RI_WAVE - 1)) < GLA_COLS) part[blk & 1][n][wave][c] = o;
+        }
+        put((blk + 1) & 1);
+        __syncthreads();
+        if (tid < nb * GLA_COLS) {
+            const int n = tid / GLA_COLS, cc = tid % GLA_COLS;
+            if (tb + n < t1 && col0 + cc < vdim) {
+                const float (*p)[GLA_COLS] = part[blk & 1][n];
+                out[((size_t)(tb + n) * heads + h) * vdim + col0 + cc] = ((p[0][cc] + p[1][cc]) + p[2][cc]) + p[3][cc];
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < GLA_MAX_ROWS; ++j) {
+        const int i = r + j * GLA_SLICES;
+        if (live && i < dim) S[(size_t)i * vdim] = s[j];
+    }
+}
+
+extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off,
+                           const float* z, const float* z_bias, float tau, float q_scale, float* state,
+                           const int32_t* cu_seqlens, const int32_t* slots, int seqs, int heads, int dim, int vdim,
+                           void* stream) {
+    RI_REQUIRE(seqs > 0 && heads > 0 && dim > 0 && vdim > 0, "gla_scan: %d sequences, %d heads of %d x %d", seqs, heads, dim, vdim);
+    RI_REQUIRE(dim <= GLA_SLICES * GLA_MAX_ROWS, "gla_scan: key heads of %d exceed the kernel's %d", dim, GLA_SLICES * GLA_MAX_ROWS);
+    RI_REQUIRE(heads <= 65535 && seqs <= 65535, "gla_scan: %d heads of %d sequences exceed one launch", heads, seqs);
+    RI_REQUIRE(tau > 0.f, "gla_scan: tau %g must be positive", (double)tau);
+    RI_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + heads * dim <= row && k_off + heads * dim <= row &&
+               v_off + heads * vdim <= row, "gla_scan: q, k, v at %d, %d, %d do not fit rows of %d", q_off, k_off, v_off, row);
+    RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "gla_scan: dtype %d", act_dtype);
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((vdim + GLA_COLS - 1) / GLA_COLS, heads, seqs);
+    int nb = GLA_STAGE * 256 / dim;
+    nb = nb > GLA_MAX_NB ? GLA_MAX_NB : nb;                  // dim <= 512: at least two tokens a block
+    const size_t lds = (size_t)2 * nb * (3 * dim + GLA_COLS) * sizeof(float);
+    if (act_dtype == RI_F32)
+        gla_scan_kernel<float><<<grid, 256, lds, s>>>(out, (const float*)proj, row, q_off, k_off, v_off, z, z_bias,
+                                                      1.0f / tau, q_scale, state, cu_seqlens, slots, heads, dim, vdim, nb);
+    else
+        gla_scan_kernel<bf16_t><<<grid, 256, lds, s>>>(out, (const bf16_t*)proj, row, q_off, k_off, v_off, z, z_bias,
+                                                       1.0f / tau, q_scale, state, cu_seqlens, slots, heads, dim, vdim, nb);
+    RI_LAUNCH_CHECK("gla_scan");
+    return 0;
+}
+
+// The scan's result per head through an RMS norm over vdim (one gain for all heads) and times silu(gate):
+// one wavefront per (token, head).
+#define GLA_NORM_PER_LANE 8      // vdim <= 64 * 8
+
+template <typename TA>
+__global__ void gla_norm_gate_kernel(TA* __restrict__ out, const float* __restrict__ o, const TA* __restrict__ proj,
+                                     int row, int g_off, const float* __restrict__ gain, float eps, long items,
+                                     int heads, int vdim) {
+    const int lane = threadIdx.x & (RI_WAVE - 1);
+    const long item = (long)blockIdx.x * (blockDim.x / RI_WAVE) + threadIdx.x / RI_WAVE;
+    if (item >= items) return;
+    const long t = item / heads;
+    const int h = (int)(item % heads);
+    const float* x = o + (size_t)item * vdim;
+    const TA* g = proj + (size_t)t * row + g_off + (size_t)h * vdim;
+    float v[GLA_NORM_PER_LANE];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < GLA_NORM_PER_LANE; ++j) {
+        const int i = lane + j * RI_WAVE;
+        v[j] = i < vdim ? x[i] : 0.f;
+        ss += v[j] * v[j];
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)vdim + eps);
+#pragma unroll
+    for (int j = 0; j < GLA_NORM_PER_LANE; ++j) {
+        const int i = lane + j * RI_WAVE;
+        if (i >= vdim) continue;
+        const float gate = to_f32(g[i]);
+        from_f32(out + (size_t)item * vdim + i, v[j] * inv * gain[i] * (gate / (1.0f + expf(-gate))));
+    }
+}
+
+extern "C" int ri_gla_norm_gate(void* out, const float* o, const void* proj, int act_dtype, int row, int g_off,
+                                const float* gain, float eps, int tokens, int heads, int vdim, void* stream) {
+    RI_REQUIRE(tokens > 0 && heads > 0 && vdim > 0 && vdim <= RI_WAVE * GLA_NORM_PER_LANE,
+               "gla_norm_gate: %d tokens, %d heads of %d", tokens, heads, vdim);
+    RI_REQUIRE(g_off >= 0 && g_off + heads * vdim <= row, "gla_norm_gate: the gate at %d does not fit rows of %d", g_off, row);
+    RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "gla_norm_gate: dtype %d", act_dtype);
+    const long items = (long)tokens * heads;
+    const long blocks = (items + 3) / 4;
+    RI_REQUIRE(blocks <= 2147483647L, "gla_norm_gate: %ld heads exceed one launch", items);
+    hipStream_t s = (hipStream_t)stream;
+    if (act_dtype == RI_F32)
+        gla_norm_gate_kernel<float><<<(unsigned)blocks, 256, 0, s>>>((float*)out, o, (const float*)proj, row, g_off, gain, eps,
+                                                                     items, heads, vdim);
+    else
+        gla_norm_gate_kernel<bf16_t><<<(unsigned)blocks, 256, 0, s>>>((bf16_t*)out, o, (const bf16_t*)proj, row, g_off, gain,
+                                                                      eps, items, heads, vdim);
+    RI_LAUNCH_CHECK("gla_norm_gate");
+    return 0;
+}

@@ -313,6 +313,46 @@ extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int in
     return 0;
 }
 
+// ------------------------------------------------------------------ squared ReLU
+// out[i] = max(y[i], 0)^2, the square taken in float32.
+template <typename T>
+__global__ void relu_squared_kernel(T* __restrict__ out, const T* __restrict__ y, long total) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    const float v = fmaxf(to_f32(y[e]), 0.f);
+    from_f32(out + e, v * v);
+}
+
+__global__ void relu_squared_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ y, long total8) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total8) return;
+    const uint4 g = *reinterpret_cast<const uint4*>(y + e * 8);
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float a = fmaxf(__uint_as_float(gw[k] << 16), 0.f), b = fmaxf(__uint_as_float(gw[k] & 0xFFFF0000u), 0.f);
+        o[k] = pack_bf16x2(a * a, b * b);
+    }
+    *reinterpret_cast<uint4*>(out + e * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+extern "C" int ri_relu_squared(void* out, const void* y, int dtype, long total, void* stream) {
+    RI_REQUIRE(total > 0, "relu_squared: %ld elements", total);
+    RI_REQUIRE((total + 255) / 256 <= 2147483647L, "relu_squared: %ld elements exceed one launch", total);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == RI_F32)
+        relu_squared_kernel<float><<<(unsigned)((total + 255) / 256), 256, 0, s>>>((float*)out, (const float*)y, total);
+    else if (dtype == RI_BF16 && total % 8 == 0 && (uintptr_t)y % 16 == 0 && (uintptr_t)out % 16 == 0)
+        relu_squared_bf16x8_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, total / 8);
+    else if (dtype == RI_BF16)
+        relu_squared_kernel<bf16_t><<<(unsigned)((total + 255) / 256), 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, total);
+    else
+        RI_REQUIRE(false, "relu_squared: dtype %d", dtype);
+    RI_LAUNCH_CHECK("relu_squared");
+    return 0;
+}
+
 // ------------------------------------------------------------------ bias
 // x[t, i] += bias[i] in place, the sum in float32 (for parts with biased products; the reference's family
 // has none: src/models/qwen3.rs:60-69).

@@ -39,7 +39,7 @@ class PlainEngine:
             n = g.need
             for e in g.entries:
                 k = np.zeros((g.pool.num_pages, n.kv_heads, g.page_size, n.head_dim), dtype=np.float32)
-                v = np.zeros((g.pool.num_pages, n.kv_heads, n.head_dim, g.page_size), dtype=np.float32)
+                v = np.zeros((g.pool.num_pages, n.kv_heads, n.value_dim, g.page_size), dtype=np.float32)
                 self.stores[e] = ((k, v), gi)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:

@@ -27,7 +27,19 @@ _SIGNATURES = {
                                  c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                  c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
-                     c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
+    "ri_qk_norm_temper_kv_write": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_float, c_int, c_void_p, c_void_p,
+                                   c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                   c_void_p],
+    "ri_streams_read_norm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p,
+                             c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_int, c_int, c_void_p],
+    "ri_embed_positions_norm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                c_int, c_int, c_int, c_void_p],
+    "ri_gla_scan": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float,
+                    c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_gla_norm_gate": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_int, c_int, c_int,
+                         c_void_p],
+    "ri_relu_squared": [c_void_p, c_void_p, c_int, ctypes.c_long, c_void_p],
     "ri_attention_prefill_bf16": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "ri_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -272,15 +284,126 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, 
 
 
 def attention(qkv, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, kv_heads: int, head_dim: int,
-              window: int | None, scale: float) -> torch.Tensor:
-    """Attention of every new token over its sequence's pages; q is the first ``H dh`` columns of ``qkv``."""
+              window: int | None, scale: float, softcap: float | None = None) -> torch.Tensor:
+    """Attention of every new token over its sequence's pages; q is the first ``H dh`` columns of ``qkv``.
+    The size of a value head is read from ``v_pages [pages, kv_heads, v_dim, page]``; with ``softcap`` a score
+    ``s`` becomes ``softcap * tanh(s / softcap)`` before the softmax."""
     tokens, stride = qkv.shape
-    out = torch.empty((tokens, heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    v_dim = v_pages.shape[2]
+    if tuple(k_pages.shape[:2]) != tuple(v_pages.shape[:2]) or k_pages.shape[2] != v_pages.shape[3] or k_pages.shape[3] != head_dim:
+        raise ShapeError(f"attention: key pages {list(k_pages.shape)} and value pages {list(v_pages.shape)} for heads of {head_dim}")
+    out = torch.empty((tokens, heads * v_dim), dtype=qkv.dtype, device=qkv.device)
     _call("ri_attention", _dev(out, "out"), _dev(qkv, "qkv"), code(qkv.dtype), stride, _dev(k_pages, "k_pages"),
           _dev(v_pages, "v_pages"), code(k_pages.dtype), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
           _dev(tok_seq, "tok_seq", torch.int32, (tokens,)), _dev(page_table, "page_table", torch.int32),
-          page_table.shape[1], tokens, heads, kv_heads, head_dim, k_pages.shape[2], int(window or 0), float(scale),
+          page_table.shape[1], tokens, heads, kv_heads, head_dim, v_dim, k_pages.shape[2], int(window or 0),
+          float(scale), float(softcap or 0.0), _stream())
+    return out
+
+
+def qk_norm_temper_kv_write(qkv, q_gain, k_gain, eps: float, temper, tok_pos, tok_seq, page_table, k_pages, v_pages,
+                            heads: int, kv_heads: int, dim: int, vdim: int) -> None:
+    """Per-head RMS norm of q and k (gains may be None), the query temperature ``temper = (coef, every)`` or None
+    (``q *= 1 + coef * ln(floor((pos + 1) / every) + 1)``, q in place), k and v into their pages.
+    ``qkv: [T, heads * dim + kv_heads * dim + kv_heads * vdim]``."""
+    tokens, stride = qkv.shape
+    if stride != (heads + kv_heads) * dim + kv_heads * vdim:
+        raise ShapeError(f"qkv rows of {stride} for {heads} + {kv_heads} heads of {dim} and {kv_heads} of {vdim}")
+    pages, _, page_size, _ = k_pages.shape
+    coef, every = (float(temper[0]), int(temper[1])) if temper else (0.0, 1)
+    _call("ri_qk_norm_temper_kv_write", _dev(qkv, "qkv"), code(qkv.dtype), _opt(q_gain, "q_gain", torch.float32, (dim,)),
+          _opt(k_gain, "k_gain", torch.float32, (dim,)), float(eps), coef, every,
+          _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1],
+          _dev(k_pages, "k_pages", None, (pages, kv_heads, page_size, dim)),
+          _dev(v_pages, "v_pages", k_pages.dtype, (pages, kv_heads, vdim, page_size)), code(k_pages.dtype),
+          tokens, heads, kv_heads, dim, vdim, page_size, _stream())
+
+
+NORM_NONE, NORM_RMS, NORM_LAYER = 0, 1, 2
+MAX_STREAMS = 8
+
+
+def streams_read_norm(streams, pending, mix, out_coef, in_coef, gain, bias, eps: float, norm_kind: int, out_dtype,
+                      rows: torch.Tensor | None = None, fresh: torch.Tensor | None = None) -> torch.Tensor:
+    """The write that waits for the residual streams, the read and the norm, in one kernel.
+    ``streams: [T, S, dim]`` float32.  With ``pending`` (``[T, dim]`` or ``[parts, T, dim]``):
+    ``x_t <- sum_s mix[s, t] x_s + out_coef[t] * pending``; then ``u = sum_t in_coef[t] x_t`` and the norm of ``u``
+    (``NORM_NONE``, ``NORM_RMS`` or ``NORM_LAYER`` with ``gain`` and optional ``bias``).  Coefficients that are
+    None are the identity and ones.  With ``rows`` only those rows are read and nothing is stored.  ``fresh``
+    (``[T, dim]``): the one row all streams start from, spread into ``streams`` by this call."""
+    t, n, dim = streams.shape
+    count = t if rows is None else rows.shape[0]
+    parts = 1
+    if pending is not None:
+        if pending.dim() == 3:
+            parts = pending.shape[0]
+        if tuple(pending.shape[-2:]) != (t, dim):
+            raise ShapeError(f"pending is {list(pending.shape)}, the streams are {list(streams.shape)}")
+    out = torch.empty((count, dim), dtype=out_dtype, device=streams.device)
+    if count == 0:
+        return out
+    _call("ri_streams_read_norm", _dev(out, "out"), code(out_dtype), _dev(streams, "streams", torch.float32),
+          _opt(fresh, "fresh", torch.float32, (t, dim)), n,
+          _opt(pending, "pending"), code(pending.dtype) if pending is not None else F32, parts, t,
+          _opt(mix, "mix", torch.float32, (n, n)), _opt(out_coef, "out_coef", torch.float32, (n,)),
+          _opt(in_coef, "in_coef", torch.float32, (n,)), _opt(gain, "gain", torch.float32, (dim,)),
+          _opt(bias, "bias", torch.float32, (dim,)), float(eps), int(norm_kind),
+          _opt(rows, "rows", torch.int32), count, dim, _stream())
+    return out
+
+
+def embed_positions_norm(table, positions, ids, tok_pos, gain, bias, eps: float, norm_kind: int) -> torch.Tensor:
+    """float32 rows ``norm(table[ids] + positions[tok_pos])`` (``positions`` may be None)."""
+    tokens, dim = ids.shape[0], table.shape[1]
+    out = torch.empty((tokens, dim), dtype=torch.float32, device=table.device)
+    if positions is not None and (positions.dtype != table.dtype or positions.shape[1] != dim):
+        raise ShapeError("the table of positions must have the token table's dtype and width")
+    _call("ri_embed_positions_norm", _dev(out, "out"), _dev(table, "table"), _opt(positions, "positions"),
+          code(table.dtype), _dev(ids, "ids", torch.int32, (tokens,)), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
+          _opt(gain, "gain", torch.float32, (dim,)), _opt(bias, "bias", torch.float32, (dim,)), float(eps),
+          int(norm_kind), tokens, dim, _stream())
+    return out
+
+
+GLA_MAX_DIM = 512
+
+
+def gla_scan(proj, q_off: int, k_off: int, v_off: int, z, z_bias, tau: float, q_scale: float, state, cu_seqlens,
+             slots, heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """The gated linear recurrence over every sequence's new tokens; float32 ``[T, heads * vdim]``.
+    ``proj: [T, row]`` holds q, k (``heads * dim``) and v (``heads * vdim``) at the given columns; ``z``
+    (float32 ``[T, heads * dim]``) and ``z_bias`` give the decay ``exp(log_sigmoid(z + bias) / tau)``;
+    ``state: [slots, heads, dim, vdim]`` float32 is read and written at the sequences' slots."""
+    tokens, row = proj.shape
+    seqs = slots.shape[0]
+    if state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, vdim):
+        raise ShapeError(f"the state is {list(state.shape)}, not [slots, {heads}, {dim}, {vdim}]")
+    out = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=proj.device)
+    _call("ri_gla_scan", _dev(out, "out"), _dev(proj, "proj"), code(proj.dtype), row, q_off, k_off, v_off,
+          _dev(z, "z", torch.float32, (tokens, heads * dim)), _opt(z_bias, "z_bias", torch.float32, (heads * dim,)),
+          float(tau), float(q_scale), _dev(state, "state", torch.float32),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
+          seqs, heads, dim, vdim, _stream())
+    return out
+
+
+def gla_norm_gate(o, proj, g_off: int, gain, eps: float, heads: int, vdim: int) -> torch.Tensor:
+    """``rms_norm(o[t, h]) * gain * silu(gate[t, h])`` in the dtype of ``proj``, whose rows hold the gate at column
+    ``g_off``; ``o``: float32 ``[T, heads * vdim]``."""
+    tokens, row = proj.shape
+    out = torch.empty((tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
+    _call("ri_gla_norm_gate", _dev(out, "out"), _dev(o, "o", torch.float32, (tokens, heads * vdim)), _dev(proj, "proj"),
+          code(proj.dtype), row, g_off, _dev(gain, "gain", torch.float32, (vdim,)), float(eps), tokens, heads, vdim,
           _stream())
+    return out
+
+
+def relu_squared(y: torch.Tensor) -> torch.Tensor:
+    """``max(y, 0)^2`` elementwise."""
+    out = torch.empty(y.shape, dtype=y.dtype, device=y.device)
+    if y.numel():
+        _call("ri_relu_squared", _dev(out, "out"), _dev(y, "y"), code(y.dtype), y.numel(), _stream())
     return out
 
 

@@ -38,13 +38,23 @@ class GroupedQueryAttention(Mixer):
     ``qkv_bias`` and ``o_bias`` add ``{q,k,v}_proj.bias`` and ``o_proj.bias`` to the products (the
     reference's family has no bias anywhere, src/models/qwen3.rs:60-69; families that differ from it in
     this alone need no other mixer).  A biased output product adds into the stream the plain way.
+
+    For families without a rotation whose attention differs in its constants: ``v_dim`` is the size of a value
+    head where it is not ``head_dim`` (the output product then reads ``heads * v_dim``); ``scale`` replaces
+    ``1 / sqrt(head_dim)``; ``softcap = c`` turns a score ``s`` into ``c tanh(s / c)`` before the softmax;
+    ``q_temper = (coef, every)`` multiplies the normed query at position ``p`` by
+    ``1 + coef * ln(floor((p + 1) / every) + 1)``, all in float32.  ``names`` gives the checkpoint names of
+    ``q, k, v, o, q_norm, k_norm`` where they are not ``<prefix>q_proj.weight`` and so on.  A mixer with any of
+    ``v_dim``, ``softcap`` or ``q_temper`` takes no position encoding; its q/k norm, temperature and cache write
+    are one kernel (``ops.qk_norm_temper_kv_write``).
     """
 
     links_norms = True
 
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, prefix: str, qk_norm: bool = True,
                  eps: float = 1e-6, position: PartSpec | None = None, window: int | None = None,
-                 qkv_bias: bool = False, o_bias: bool = False):
+                 qkv_bias: bool = False, o_bias: bool = False, v_dim: int | None = None, scale: float | None = None,
+                 softcap: float | None = None, q_temper: tuple | None = None, names: dict | None = None):
         if heads < 1 or kv_heads < 1 or heads % kv_heads:
             raise ConfigError(f"{heads} attention heads not divisible by {kv_heads} kv heads")
         if not 1 <= head_dim <= ops.MAX_HEAD_DIM:
@@ -54,20 +64,39 @@ class GroupedQueryAttention(Mixer):
         self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim
         self.prefix, self.qk_norm, self.eps, self.window = prefix, qk_norm, eps, window
         self.qkv_bias, self.o_bias = qkv_bias, o_bias
-        self.scale = 1.0 / math.sqrt(head_dim)                      # src/attention.rs:28
+        self.scale = 1.0 / math.sqrt(head_dim) if scale is None else float(scale)      # src/attention.rs:28
+        self.v_dim = head_dim if v_dim is None else int(v_dim)
+        self.softcap = float(softcap) if softcap else None
+        self.q_temper = (float(q_temper[0]), int(q_temper[1])) if q_temper else None
+        if not 1 <= self.v_dim <= ops.MAX_HEAD_DIM:
+            raise ConfigError(f"value heads of {self.v_dim}: the attention kernels take 1 to {ops.MAX_HEAD_DIM}")
+        if self.q_temper is not None and self.q_temper[1] < 1:
+            raise ConfigError(f"a query temperature every {self.q_temper[1]} positions")
+        # what the rotary kernels do not know goes through the kernels that do
+        self.tempered = self.v_dim != head_dim or self.q_temper is not None
         self.position = build_part("position", position or PartSpec("none"))
+        if (self.tempered or self.softcap is not None) and (position is not None and position.kind != "none"):
+            raise ConfigError("an attention with a score cap, a query temperature or value heads of their own size "
+                              "takes no position encoding")
+        if (self.tempered or self.softcap is not None) and (qkv_bias or o_bias):
+            raise ConfigError("an attention with a score cap, a query temperature or value heads of their own size "
+                              "takes no biases")
+        p = prefix
+        self.names = {"q": p + "q_proj.weight", "k": p + "k_proj.weight", "v": p + "v_proj.weight",
+                      "o": p + "o_proj.weight", "q_norm": p + "q_norm.weight", "k_norm": p + "k_norm.weight"}
+        self.names.update(names or {})
 
     def tensors(self):
-        p, d, dh = self.prefix, self.hidden, self.head_dim
+        p, d, dh, n = self.prefix, self.hidden, self.head_dim, self.names
         t = {
-            p + "q_proj.weight": TensorSpec((self.heads * dh, d), MATRIX),
-            p + "k_proj.weight": TensorSpec((self.kv_heads * dh, d), MATRIX),
-            p + "v_proj.weight": TensorSpec((self.kv_heads * dh, d), MATRIX),
-            p + "o_proj.weight": TensorSpec((d, self.heads * dh), MATRIX),
+            n["q"]: TensorSpec((self.heads * dh, d), MATRIX),
+            n["k"]: TensorSpec((self.kv_heads * dh, d), MATRIX),
+            n["v"]: TensorSpec((self.kv_heads * self.v_dim, d), MATRIX),
+            n["o"]: TensorSpec((d, self.heads * self.v_dim), MATRIX),
         }
         if self.qk_norm:
-            t[p + "q_norm.weight"] = TensorSpec((dh,), GAIN)
-            t[p + "k_norm.weight"] = TensorSpec((dh,), GAIN)
+            t[n["q_norm"]] = TensorSpec((dh,), GAIN)
+            t[n["k_norm"]] = TensorSpec((dh,), GAIN)
         if self.qkv_bias:
             t[p + "q_proj.bias"] = TensorSpec((self.heads * dh,), BIAS)
             t[p + "k_proj.bias"] = TensorSpec((self.kv_heads * dh,), BIAS)
@@ -79,12 +108,12 @@ class GroupedQueryAttention(Mixer):
 
     def bind(self, weights, rt):
         self.rt = rt
-        p = self.prefix
-        qkv = torch.cat([weights[p + "q_proj.weight"], weights[p + "k_proj.weight"], weights[p + "v_proj.weight"]], 0)
+        p, n = self.prefix, self.names
+        qkv = torch.cat([weights[n["q"]], weights[n["k"]], weights[n["v"]]], 0)
         self.w_qkv = rt.pack(rt.place_matrix(qkv))
-        self.w_o = rt.pack(rt.place_matrix(weights[p + "o_proj.weight"]), parts_ok=(p + "o_proj.bias") not in weights)
-        self.q_gain = rt.place_gain(weights[p + "q_norm.weight"]) if self.qk_norm else None
-        self.k_gain = rt.place_gain(weights[p + "k_norm.weight"]) if self.qk_norm else None
+        self.w_o = rt.pack(rt.place_matrix(weights[n["o"]]), parts_ok=(p + "o_proj.bias") not in weights)
+        self.q_gain = rt.place_gain(weights[n["q_norm"]]) if self.qk_norm else None
+        self.k_gain = rt.place_gain(weights[n["k_norm"]]) if self.qk_norm else None
         self.b_qkv = self.b_o = None
         if self.qkv_bias:
             self.b_qkv = rt.place_gain(torch.cat([weights[p + n + "_proj.bias"] for n in "qkv"], 0))
@@ -93,9 +122,12 @@ class GroupedQueryAttention(Mixer):
         self.position.bind(weights, rt)
 
     def bind_plain(self, weights):
+        if self.tempered or self.softcap is not None:
+            raise ConfigError("an attention with a score cap, a query temperature or value heads of their own size has "
+                              "no plain form")
         f32 = lambda name: weights[self.prefix + name].to(torch.float32).numpy()
-        self.plain_w = {n: f32(n + "_proj.weight") for n in "qkvo"}
-        self.plain_gain = {n: f32(n + "_norm.weight") for n in "qk"} if self.qk_norm else {}
+        self.plain_w = {n: weights[self.names[n]].to(torch.float32).numpy() for n in "qkvo"}
+        self.plain_gain = {n: weights[self.names[n + "_norm"]].to(torch.float32).numpy() for n in "qk"} if self.qk_norm else {}
         self.plain_bias = {n: f32(n + "_proj.bias") for n in ("qkv" if self.qkv_bias else "") + ("o" if self.o_bias else "")}
         if getattr(self.position, "acts_after_norm", False) or not hasattr(self.position, "plain"):
             raise ConfigError(f"the position encoding {type(self.position).__name__} has no plain form")
@@ -129,7 +161,7 @@ class GroupedQueryAttention(Mixer):
         return self.rt.takes_tiled(self.w_qkv, m)
 
     def cache_need(self):
-        return KVNeed(self.kv_heads, self.head_dim, self.window)
+        return KVNeed(self.kv_heads, self.head_dim, self.window, None if self.v_dim == self.head_dim else self.v_dim)
 
     def forward(self, x, ctx, store, page_table, link=None):
         rt = self.rt
@@ -137,6 +169,8 @@ class GroupedQueryAttention(Mixer):
             qkv = rt.linear_packed(x, self.w_qkv)
             if self.b_qkv is not None:
                 ops.add_bias(qkv, self.b_qkv)
+        if self.tempered or self.softcap is not None:
+            return self.forward_tempered(qkv, ctx, store, page_table, link)
         self.position.apply(qkv, ctx, self.heads, self.kv_heads, self.head_dim)
         group = self.heads // self.kv_heads
         table = self.position.rotation_table()
@@ -172,6 +206,18 @@ class GroupedQueryAttention(Mixer):
                                           page_table, store.k_pages, store.v_pages, *shape, ctx.cu_seqlens, ctx.max_new)
         with profiler.section(profiler.ATTENTION):
             o = self.attend(qkv, ctx, store, page_table)
+        return self.project_out(o, link)
+
+    def forward_tempered(self, qkv, ctx, store, page_table, link):
+        """No rotation: per-head norm, query temperature and the write of k and v in one kernel, then the attention
+        with the score cap."""
+        with profiler.section(profiler.QK_NORM_ROPE_APPEND):
+            ops.qk_norm_temper_kv_write(qkv, self.q_gain, self.k_gain, self.eps, self.q_temper, ctx.tok_pos, ctx.tok_seq,
+                                        page_table, store.k_pages, store.v_pages, self.heads, self.kv_heads,
+                                        self.head_dim, self.v_dim)
+        with profiler.section(profiler.ATTENTION):
+            o = ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads,
+                              self.kv_heads, self.head_dim, self.window, self.scale, self.softcap)
         return self.project_out(o, link)
 
     def project_out(self, o, link):

@@ -41,6 +41,10 @@ class ResidualStream:
         self.next_entry_tiled = False  # and whether the part behind it reads tiled rows
         self.links_ok = True         # whether norms may be left to products at all (not where every step must run alike)
 
+    @property
+    def rows(self) -> int:
+        return self.sum.shape[0]
+
     def link(self, norm, act_dtype, tiled: bool = False):
         """A ``NormLink`` for the branch that is about to run, if ``norm`` is the next reader of the
         stream and can be left to a product.  ``tiled``: the part behind that norm reads tiled rows."""
@@ -102,11 +106,15 @@ class PreNormBlock:
     def __init__(self, layer_spec):
         self.mixer_norm = build_part("norm", layer_spec.mixer_norm)
         self.mixer = build_part("mixer", layer_spec.mixer)
-        self.feed_forward_norm = build_part("norm", layer_spec.feed_forward_norm)
-        self.feed_forward = build_part("feed_forward", layer_spec.feed_forward)
+        # a layer without a feed-forward names neither it nor its norm: it is the first sublayer alone
+        self.feed_forward_norm = self.feed_forward = None
+        if "feed_forward" in layer_spec.parts:
+            self.feed_forward_norm = build_part("norm", layer_spec.feed_forward_norm)
+            self.feed_forward = build_part("feed_forward", layer_spec.feed_forward)
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
+        both = (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
+        return both if self.feed_forward is not None else both[:2]
 
     def entry_norm(self):
         """The norm through which this layer first reads the stream."""
@@ -119,18 +127,24 @@ class PreNormBlock:
     def plain(self, h, ctx, store, page_table):
         """``h`` after this layer, float32 numpy (the plain backend)."""
         r = h + self.mixer.plain(self.mixer_norm.plain(h), ctx, store, page_table)
+        if self.feed_forward is None:
+            return r
         return r + self.feed_forward.plain(self.feed_forward_norm.plain(r), ctx)
 
     def forward(self, stream: ResidualStream, ctx, store, page_table, act_dtype) -> None:
         # a part with ``links_norms`` takes a NormedLater as input and a NormLink for its output
         rows = stream.sum.shape[0]
+        after_mixer = self.feed_forward_norm if self.feed_forward is not None else stream.next_entry_norm
         if getattr(self.mixer, "links_norms", False):
             h = stream.normed(self.mixer_norm, act_dtype, later_ok=True, tiled=_takes_tiled(self.mixer, rows))
-            link = stream.link(self.feed_forward_norm, act_dtype, _takes_tiled(self.feed_forward, rows))
+            link = stream.link(after_mixer, act_dtype, _takes_tiled(self.feed_forward, rows) if self.feed_forward is not None
+                               else stream.next_entry_tiled)
             stream.push(self.mixer.forward(h, ctx, store, page_table, link=link))
         else:
             h = stream.normed(self.mixer_norm, act_dtype)
             stream.push(self.mixer.forward(h, ctx, store, page_table))
+        if self.feed_forward is None:
+            return
         if getattr(self.feed_forward, "links_norms", False):
             h = stream.normed(self.feed_forward_norm, act_dtype, later_ok=True,
                               tiled=_takes_tiled(self.feed_forward, rows))
@@ -139,3 +153,34 @@ class PreNormBlock:
         else:
             h = stream.normed(self.feed_forward_norm, act_dtype)
             stream.push(self.feed_forward.forward(h, ctx))
+
+
+@register_part("arrangement", "hyper_prenorm")
+class HyperConnectedBlock:
+    """The pre-norm layer over a residual kept in several streams (``parts.streams.HyperStream``): each
+    sublayer reads the streams through its connection's ``in`` coefficients and its norm, and its output is
+    written to all streams through ``mix`` and ``out``.  Parts: ``mixer_norm``, ``mixer``, ``mixer_connection``
+    and, for a layer that has a feed-forward, ``feed_forward_norm``, ``feed_forward``, ``feed_forward_connection``."""
+
+    def __init__(self, layer_spec):
+        self.mixer_norm = build_part("norm", layer_spec.mixer_norm)
+        self.mixer = build_part("mixer", layer_spec.mixer)
+        self.mixer_connection = build_part("connection", layer_spec.mixer_connection)
+        self.feed_forward_norm = self.feed_forward = self.feed_forward_connection = None
+        if "feed_forward" in layer_spec.parts:
+            self.feed_forward_norm = build_part("norm", layer_spec.feed_forward_norm)
+            self.feed_forward = build_part("feed_forward", layer_spec.feed_forward)
+            self.feed_forward_connection = build_part("connection", layer_spec.feed_forward_connection)
+
+    def parts(self):
+        first = (self.mixer_norm, self.mixer, self.mixer_connection)
+        if self.feed_forward is None:
+            return first
+        return first + (self.feed_forward_norm, self.feed_forward, self.feed_forward_connection)
+
+    def forward(self, stream, ctx, store, page_table, act_dtype) -> None:
+        h = stream.read(self.mixer_connection, self.mixer_norm, act_dtype)
+        stream.write(self.mixer.forward(h, ctx, store, page_table), self.mixer_connection)
+        if self.feed_forward is not None:
+            h = stream.read(self.feed_forward_connection, self.feed_forward_norm, act_dtype)
+            stream.write(self.feed_forward.forward(h, ctx), self.feed_forward_connection)

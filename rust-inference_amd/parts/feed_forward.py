@@ -4,6 +4,7 @@ from __future__ import annotations
 import torch
 
 from .. import profiler
+from ..kernels import ops
 from ..weights.loader import MATRIX, TensorSpec
 from .base import FeedForward
 from .registry import register_part
@@ -57,3 +58,29 @@ class SwiGLU(FeedForward):
             a = rt.linear_packed(x, self.w_gate_up, tiled_out=rt.takes_tiled(self.w_down, x.shape[0], True))
             # may come in parts: the stream's next norm adds them
             return rt.linear_packed(a, self.w_down, parts_ok=True, link=link)
+
+
+@register_part("feed_forward", "relu2")
+class ReluSquaredFF(FeedForward):
+    """``down(relu(up(x))^2)``, no gate and no bias; ``names`` gives the checkpoint names of ``up`` and ``down``
+    where they are not ``<prefix>up_proj.weight`` and ``<prefix>down_proj.weight``."""
+
+    def __init__(self, hidden: int, inter: int, prefix: str, names: dict | None = None):
+        self.hidden, self.inter, self.prefix = hidden, inter, prefix
+        self.names = {"up": prefix + "up_proj.weight", "down": prefix + "down_proj.weight"}
+        self.names.update(names or {})
+
+    def tensors(self):
+        return {self.names["up"]: TensorSpec((self.inter, self.hidden), MATRIX),
+                self.names["down"]: TensorSpec((self.hidden, self.inter), MATRIX)}
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.w_up = rt.pack(rt.place_matrix(weights[self.names["up"]]))
+        self.w_down = rt.pack(rt.place_matrix(weights[self.names["down"]]), parts_ok=True)
+
+    def forward(self, x, ctx):
+        rt = self.rt
+        with profiler.section(profiler.MLP):
+            a = ops.relu_squared(ops.as_rows(rt.linear_packed(x, self.w_up)))
+            return rt.linear_packed(a, self.w_down, parts_ok=True)      # may come in parts: the stream's next read adds them

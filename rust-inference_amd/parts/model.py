@@ -45,6 +45,42 @@ class TokenEmbedding(Embedding):
         return plain.embedding(self.table_plain, ctx.tokens)
 
 
+@register_part("embedding", "table_positions")
+class PositionedEmbedding(Embedding):
+    """``h[t, :] = norm(E[id_t, :] + P[pos_t, :])``: a learned row per position added to the token's row (neither
+    scaled), then an optional norm (a ``PartSpec`` of the norm category), in one kernel.  Positions count from 0
+    in every sequence and must stay below the table's ``max_positions``: a cache made for the model holds no
+    sequence longer than that."""
+
+    def __init__(self, vocab: int, dim: int, max_positions: int, name: str, positions_name: str, norm=None):
+        self.vocab, self.dim, self.max_positions = vocab, dim, max_positions
+        self.name, self.positions_name = name, positions_name
+        self.norm = build_part("norm", norm) if norm is not None else None
+
+    def tensors(self):
+        t = {self.name: TensorSpec((self.vocab, self.dim), MATRIX),
+             self.positions_name: TensorSpec((self.max_positions, self.dim), MATRIX)}
+        if self.norm is not None:
+            t.update(self.norm.tensors())
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.table = rt.place_matrix(weights[self.name])
+        self.positions = rt.place_matrix(weights[self.positions_name]).to(self.table.dtype)
+        if self.norm is not None:
+            self.norm.bind(weights, rt)
+
+    def forward(self, ctx):
+        longest = max(s + n for s, n in zip(ctx.starts, ctx.new_counts)) if ctx.starts else 0
+        if longest > self.max_positions and not torch.cuda.is_current_stream_capturing():
+            raise ShapeError(f"a sequence of {longest} tokens exceeds the {self.max_positions} positions the model has")
+        n = self.norm
+        return ops.embed_positions_norm(self.table, self.positions, ctx.tokens, ctx.tok_pos,
+                                        n.gain if n is not None else None, getattr(n, "bias", None),
+                                        n.eps if n is not None else 0.0, n.kind if n is not None else ops.NORM_NONE)
+
+
 @register_part("head", "linear")
 class OutputHead(Head):
     """``logits = x W^T`` in float32, no scaling or cap.  The matrix is the embedding
@@ -133,6 +169,7 @@ class DecoderModel:
         self.layers = [part_class("arrangement", ls.arrangement)(ls) for ls in spec.layers]
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
+        self.stream_kind = getattr(spec, "stream", None)
         self.schedule = list(spec.schedule)
         for r in self.schedule:
             if not 0 <= r.layer < len(self.layers):
@@ -228,6 +265,9 @@ class DecoderModel:
         # the configuration's max_position_embeddings is the default length only: nothing in this
         # architecture depends on it (the reference reads it and never uses it, src/models/config.rs:30)
         max_seq_len = max_seq_len or self.spec.max_positions
+        learned = getattr(self.embedding, "max_positions", None)      # a table of positions bounds every sequence
+        if learned is not None:
+            max_seq_len = min(max_seq_len, learned)
         return Cache(self.cache_needs(), num_slots, max_tokens, max_seq_len, dtype=self.rt.dtype,
                      device=self.rt.device, **kw)
 
@@ -236,15 +276,19 @@ class DecoderModel:
         """float32 logits ``[n_want, vocab]`` for the wanted rows of this step's tokens."""
         rt = self.rt
         with profiler.section(profiler.EMBEDDING):
-            stream = ResidualStream(self.embedding.forward(ctx))
-        stream.links_ok = not rt.invariant
+            hidden = self.embedding.forward(ctx)
+        if self.stream_kind is None or self.stream_kind.kind == "residual":
+            stream = ResidualStream(hidden)
+            stream.links_ok = not rt.invariant
+        else:
+            stream = part_class("stream", self.stream_kind.kind)(hidden, **self.stream_kind.params)
         for at, run in enumerate(self.schedule):
             layer = self.layers[run.layer]
             follower = self.layers[self.schedule[at + 1].layer] if at + 1 < len(self.schedule) else None
             entry = getattr(follower, "entry_norm", None)
             stream.next_entry_norm = entry() if entry else None
             tiled = getattr(follower, "entry_takes_tiled", None)
-            stream.next_entry_tiled = tiled(stream.sum.shape[0]) if tiled else False
+            stream.next_entry_tiled = tiled(stream.rows) if tiled else False
             stores, tables = [], []
             for entry in run.entries():
                 need = cache.needs[entry]

@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops, plain
-from ..weights.loader import GAIN, TensorSpec
+from ..weights.loader import BIAS, GAIN, TensorSpec
 from .base import Norm
 from .registry import register_part
 
@@ -15,6 +15,7 @@ class RMSNorm(Norm):
     float32 (the reference: src/ops/norm.rs:7-32; fused with the add: :35-62)."""
 
     accepts_parts = True
+    kind = ops.NORM_RMS      # what the kernel that also writes and reads several residual streams calls this norm
     linkable = True          # gain, eps and dim are all a product needs to do this norm itself
     can_tile = True          # hands its rows on in the matrix cores' order when asked (up to 64 rows)
 
@@ -37,3 +38,33 @@ class RMSNorm(Norm):
     def apply(self, residual, pending, out_dtype, rows=None, tiled=False):
         tiled = tiled and self.dim % 4 == 0 and self.dim <= 8192        # what the vectorised kernel takes
         return ops.add_rmsnorm(residual, pending, self.gain, self.eps, out_dtype, rows, tiled=tiled)
+
+
+@register_part("norm", "layernorm")
+class LayerNorm(Norm):
+    """``y = (x - mean) / sqrt(var + eps) * w + b`` over the last axis, ``var`` the mean of the squared deviations,
+    statistics in float32; the bias is optional (``bias_name`` None: none).  Fused with the residual add that
+    precedes it, and, for a residual kept in several streams, with the streams' write and read
+    (``ops.streams_read_norm``)."""
+
+    accepts_parts = True
+    kind = ops.NORM_LAYER
+
+    def __init__(self, dim: int, eps: float, name: str, bias_name: str | None = None):
+        self.dim, self.eps, self.name, self.bias_name = dim, eps, name, bias_name
+
+    def tensors(self):
+        t = {self.name: TensorSpec((self.dim,), GAIN)}
+        if self.bias_name:
+            t[self.bias_name] = TensorSpec((self.dim,), BIAS)
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.gain = rt.place_gain(weights[self.name])
+        self.bias = rt.place_gain(weights[self.bias_name]) if self.bias_name else None
+
+    def apply(self, residual, pending, out_dtype, rows=None, tiled=False):
+        # one stream without coefficients: residual += pending, then the norm
+        return ops.streams_read_norm(residual.view(residual.shape[0], 1, self.dim), pending, None, None, None,
+                                     self.gain, self.bias, self.eps, self.kind, out_dtype, rows)

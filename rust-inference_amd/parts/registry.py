@@ -8,7 +8,7 @@ from __future__ import annotations
 
 from ..errors import UnsupportedError
 
-CATEGORIES = ("mixer", "feed_forward", "norm", "position", "arrangement", "embedding", "head")
+CATEGORIES = ("mixer", "feed_forward", "norm", "position", "arrangement", "embedding", "head", "stream", "connection")
 _REGISTRY: dict[str, dict[str, type]] = {c: {} for c in CATEGORIES}
 
 

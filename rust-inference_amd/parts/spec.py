@@ -83,6 +83,8 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     max_positions: int
+    # how the residual is kept between the layers: "residual" (one float32 sum) or a kind with several streams
+    stream: PartSpec = PartSpec("residual")
 
     @property
     def num_cache_entries(self) -> int:

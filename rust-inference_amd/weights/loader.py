@@ -23,11 +23,12 @@ MATRIX = "matrix"     # linear and embedding weights: N(0, 0.02) when random
 GAIN = "gain"         # norm gains: 1 + N(0, 0.1) when random; always used in 32-bit
 TABLE = "table"       # integer tables
 BIAS = "bias"         # biases of products: drawn like matrices when random, used in 32-bit like gains
+MIXING = "mixing"     # small square matrices that mix residual streams: identity + N(0, 0.1) when random; used in 32-bit
 
 
 @dataclass(frozen=True)
 class TensorSpec:
-    shape: tuple
+    shape: tuple               # a size of None is given by the file alone (a rank that no configuration key names)
     kind: str = MATRIX
     optional: bool = False     # absent is fine (e.g. lm_head.weight of a tied model)
 
@@ -43,8 +44,8 @@ def check_folder(folder: ModelFolder, expected: dict[str, TensorSpec]) -> None:
                 missing.append(name)
             continue
         info = folder.info(name)
-        if tuple(info.shape) != tuple(spec.shape):
-            misshapen.append(f"{name}: file has {list(info.shape)}, model wants {list(spec.shape)}")
+        if len(info.shape) != len(spec.shape) or any(w is not None and w != h for h, w in zip(info.shape, spec.shape)):
+            misshapen.append(f"{name}: file has {list(info.shape)}, model wants {['any' if w is None else w for w in spec.shape]}")
         if info.dtype is None:
             wrong_dtype.append(f"{name}: stored as {info.stored_as}, which this library does not read")
         elif spec.kind == TABLE:

@@ -16,7 +16,7 @@ import os
 import torch
 
 from ..config import config_from_dict
-from .loader import GAIN, MATRIX, TABLE, TensorSpec
+from .loader import GAIN, MATRIX, MIXING, TABLE, TensorSpec
 from .safetensors_io import save_file
 
 
@@ -35,6 +35,8 @@ def random_tensor(seed: int, name: str, spec: TensorSpec, dtype=torch.bfloat16, 
     x = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device)
     if spec.kind == GAIN:
         x = 1.0 + gain_std * x
+    elif spec.kind == MIXING:
+        x = torch.eye(spec.shape[0], spec.shape[1], dtype=torch.float32, device=device) + gain_std * x
     else:
         x = matrix_std * x
     return x.to(dtype)
