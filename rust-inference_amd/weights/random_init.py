@@ -29,6 +29,10 @@ def _generator(seed: int, name: str, device="cpu") -> torch.Generator:
 
 def random_tensor(seed: int, name: str, spec: TensorSpec, dtype=torch.bfloat16, device="cpu",
                   matrix_std: float = 0.02, gain_std: float = 0.1) -> torch.Tensor:
+    if any(n is None for n in spec.shape):
+        from ..errors import ConfigError
+        raise ConfigError(f"{name}: a size that only a checkpoint gives ({list(spec.shape)}); a configuration that is to be "
+                          "filled with random weights must name it (a gla mixer's 'rank')")
     g = _generator(seed, name, device)
     if spec.kind == TABLE:
         return torch.zeros(spec.shape, dtype=torch.int32, device=device)

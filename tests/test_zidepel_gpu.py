@@ -1,0 +1,250 @@
+"""The Zidepel design through the engine, against the plain implementation (tests/plain/zidepel_plain.py), in
+float32 and in bfloat16, for configurations made here with random weights: whole prompts; the last tokens one by
+one; prompts in portions down to two tokens; batches of unequal requests one after another, so that slots, pages
+and states are used again; long decoding over page borders and temperature steps; a state that must survive every
+cut; greedy generation through the library's own entry point with and without graphs; the trace program."""
+import copy
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import trace_plans as plans
+from helpers import assert_logits_close, read_model_f64, rel_to_max
+from plain import zidepel_plain as Z
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def attention(heads, kv_heads, dim, vdim, scale, softcap, q_temp, ff):
+    return {"type": "attention", "mlp": None if ff is None else {"kind": "dense", "ff": ff},
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "softcap": softcap,
+                      "q_temp": q_temp}}
+
+
+def gla(heads, dim, vdim, tau, rank, ff):
+    return {"type": "gla", "mlp": None if ff is None else {"kind": "dense", "ff": ff},
+            "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau, "rank": rank}}
+
+
+# Three streams, value heads larger than key heads, a looped stretch that holds a recurrent layer, a layer
+# without feed-forward, an attention layer with neither cap nor temperature.
+Z_A = {"architecture": "Zidepel", "vocab": 211, "width": 96, "max_positions": 600, "norm": {"eps": 1e-5}, "streams": 3,
+       "loop": {"start": 1, "stop": 3, "times": 2},
+       "layers": [attention(6, 2, 24, 40, 0.2, 6.0, {"coef": 0.5, "every": 5}, 136),
+                  gla(3, 24, 16, 4.0, 8, None),
+                  attention(4, 4, 16, 16, 0.3, None, None, 72)]}
+# One plain residual (no streams), no loop, one kv head, a temperature step at every position.
+Z_B = {"architecture": "Zidepel", "vocab": 300, "width": 64, "max_positions": 1200, "norm": {"eps": 1e-6},
+       "layers": [gla(2, 40, 24, 9.0, 5, 100),
+                  attention(2, 1, 32, 32, 0.18, 30.0, {"coef": 0.2, "every": 1}, None)]}
+# One stream with its coefficients, heads of 64 (the size the matrix cores take), a layer run three times.
+Z_C = {"architecture": "Zidepel", "vocab": 157, "width": 128, "max_positions": 400, "norm": {"eps": 1e-5}, "streams": 1,
+       "loop": {"start": 0, "stop": 1, "times": 3},
+       "layers": [attention(8, 2, 64, 64, 0.11, 12.0, {"coef": 0.3, "every": 64}, 200),
+                  gla(2, 64, 64, 16.0, 16, 96)]}
+CONFIGS = {"A": Z_A, "B": Z_B, "C": Z_C}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    from rust_inference_amd.weights import write_random_model
+    base = tmp_path_factory.mktemp("zidepel")
+    return {name: write_random_model(str(base / name), cfg, seed, torch.bfloat16, matrix_std=0.12, gain_std=0.1)
+            for seed, (name, cfg) in enumerate(CONFIGS.items())}
+
+
+_models, _plain, _read = {}, {}, {}
+
+
+def loaded(folders, name, dtype_name):
+    from rust_inference_amd.parts import load_model
+    if (name, dtype_name) not in _models:
+        _models[(name, dtype_name)] = load_model(folders[name], DTYPES[dtype_name])
+    return _models[(name, dtype_name)]
+
+
+def plain_logits(folder, tokens):
+    key = (folder, tuple(tokens))
+    if key not in _plain:
+        if folder not in _read:
+            _read[folder] = read_model_f64(folder)
+        _plain[key] = Z.logits(*_read[folder], list(tokens))
+    return _plain[key]
+
+
+def requests_for(name, lengths, seed):
+    rng = np.random.default_rng(seed)
+    return {f"{name}{i}": [int(t) for t in rng.integers(0, CONFIGS[name]["vocab"], n)] for i, n in enumerate(lengths)}
+
+
+def replay(model, steps):
+    from rust_inference_amd.engine.replay import Replayer, engine_for_trace
+    engine = engine_for_trace(model, plans.max_live_tokens(steps))
+    player = Replayer(engine)
+    outs = {}
+    for s in steps:
+        logits = player.feed(s)
+        if logits is not None:
+            outs[s["step"]] = logits.cpu().numpy()
+    engine.cache.check_consistent()
+    assert engine.cache.slots.free_count == engine.cache.num_slots
+    assert all(f == g.pool.num_pages for f, g in zip(engine.cache.free_pages(), engine.cache.groups))
+    return plans.collect(steps, lambda i: outs[i], model.spec.vocab_size)
+
+
+def against_plain(folder, got, requests, dtype_name, what):
+    for rid, toks in requests.items():
+        assert_logits_close(got[rid], plain_logits(folder, toks), dtype_name, f"{what}, request {rid}")
+
+
+def in_portions(requests, sizes):
+    """Each request alone, its prompt in portions of the given sizes in turn (the last portion takes what is left)."""
+    steps = []
+    for rid, toks in requests.items():
+        at, i = 0, 0
+        while at < len(toks):
+            n = min(sizes[i % len(sizes)], len(toks) - at)
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks[at:at + n], "want": list(range(n))}],
+                          "end": [rid] if at + n == len(toks) else []})
+            at, i = at + n, i + 1
+    return steps
+
+
+LENGTHS = {"A": [70, 3, 131], "B": [45, 1, 200], "C": [97, 33, 64]}
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_whole_prompts(folders, name, dtype_name):
+    reqs = requests_for(name, LENGTHS[name], 1)
+    got = replay(loaded(folders, name, dtype_name), plans.whole(reqs))
+    against_plain(folders[name], got, reqs, dtype_name, "whole")
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_last_tokens_one_by_one_and_portions(folders, name, dtype_name):
+    reqs = requests_for(name, [n + 40 for n in LENGTHS[name]], 2)
+    model = loaded(folders, name, dtype_name)
+    whole = replay(model, plans.whole(reqs))
+    bound = 2e-5 if dtype_name == "float32" else 2e-2
+    for what, steps in (("last 32 one by one", plans.tail_one_by_one(reqs, 32)),
+                        ("portions of 2, 31 and 32", in_portions(reqs, [2, 31, 32])),
+                        ("portions of 64, 1 and 7", in_portions(reqs, [64, 1, 7]))):
+        got = replay(model, steps)
+        against_plain(folders[name], got, reqs, dtype_name, what)
+        for rid in reqs:
+            err = rel_to_max(got[rid], whole[rid])
+            assert err <= bound, f"{rid}, {what}: differs from the whole prompt by {err:.2e} of the largest logit"
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_unequal_batches_one_after_another(folders, name, dtype_name):
+    rng = np.random.default_rng(7)
+    batches, reqs = [], {}
+    for b in range(3):                                       # three batches on one cache: slots, pages and states come back
+        batch = {}
+        for i in rng.permutation(len(LENGTHS[name])):
+            p = LENGTHS[name][i]
+            toks = [int(t) for t in rng.integers(0, CONFIGS[name]["vocab"], p + int(rng.integers(0, 14)))]
+            batch[f"{name}{b}_{i}"] = (toks, p)
+            reqs[f"{name}{b}_{i}"] = toks
+        batches.append(batch)
+    model = loaded(folders, name, dtype_name)
+    got = replay(model, plans.unequal_batches(batches))
+    against_plain(folders[name], got, reqs, dtype_name, "unequal batches")
+    alone = replay(model, plans.whole(reqs))
+    bound = 2e-5 if dtype_name == "float32" else 2e-2
+    for rid in reqs:
+        assert rel_to_max(got[rid], alone[rid]) <= bound, f"{rid}: in a batch it differs from itself alone"
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_long_decoding_from_the_first_tokens(folders, name, dtype_name):
+    """Three tokens of prompt, then 150 one by one: over page borders and many steps of the temperature."""
+    reqs = requests_for(name, [153], 3)
+    got = replay(loaded(folders, name, dtype_name), plans.tail_one_by_one(reqs, 150))
+    against_plain(folders[name], got, reqs, dtype_name, "long decoding")
+
+
+@pytest.mark.parametrize("cuts", [[300], [1] * 40 + [260], [33, 2, 265], [299, 1]])
+def test_a_state_that_hardly_decays_survives_every_cut(folders, tmp_path_factory, cuts):
+    """With the decay's bias far on the positive side the recurrent state keeps the first tokens for hundreds of
+    steps: a state that is lost, reset or carried to the wrong slot at any cut changes the last logits."""
+    from safetensors.torch import load_file, save_file
+    from rust_inference_amd.parts import load_model
+    folder = str(tmp_path_factory.mktemp("slow_decay"))
+    w = load_file(os.path.join(folders["B"], "model.safetensors"))
+    w["l0.mix.a2.b"] = torch.full_like(w["l0.mix.a2.b"], 9.0)
+    save_file(w, os.path.join(folder, "model.safetensors"))
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(Z_B, f)
+    toks = requests_for("B", [300], 4)["B0"]
+    want = plain_logits(folder, toks)
+    other = plain_logits(folder, [toks[0] ^ 1] + toks[1:])
+    assert rel_to_max(other[-1], want[-1]) > 1e-3, "the first token does not reach the last logits: the test shows nothing"
+    model = load_model(folder, torch.float32)
+    steps, at = [], 0
+    for n in cuts:
+        # another request comes and goes between the portions, on the slot next to this one
+        steps.append({"step": len(steps), "entries": [{"id": "x", "tokens": toks[at:at + n], "want": list(range(n))}], "end": []})
+        steps.append({"step": len(steps), "entries": [{"id": f"o{at}", "tokens": toks[:5], "want": []}], "end": [f"o{at}"]})
+        at += n
+    steps[-1]["end"].append("x")
+    got = replay(model, steps)
+    assert_logits_close(got["x"], want, "float32", f"cuts {cuts[:3]}")
+
+
+@pytest.mark.parametrize("dtype_name, use_graphs", [("float32", False), ("float32", True), ("bfloat16", True)])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_greedy_generation_through_the_entry_point(folders, name, dtype_name, use_graphs):
+    from rust_inference_amd import Model
+    prompts = list(requests_for(name, [33, 2, 40, 7], 5).values())
+    steps = 12
+    cfg, w = read_model_f64(folders[name])
+    model = Model.load(folders[name], dtype=dtype_name, max_batch=3, max_seq_len=128, use_graphs=use_graphs, graph_after=0)
+    got = model.generate(prompts, max_new_tokens=steps).tokens          # four prompts on three slots: a second batch
+    for g, p in zip(got, prompts):
+        toks, rows = Z.greedy(cfg, w, p, steps)
+        for i, (a, b) in enumerate(zip(g, toks)):
+            if a != b:
+                top = np.sort(rows[i])
+                assert top[-1] - top[-2] < (1e-4 if dtype_name == "float32" else 0.08), f"token {i} is {a}, plain says {b}"
+                break                                                   # from here on the two follow different texts
+    model.cache.check_consistent()
+
+
+def test_the_trace_program(folders, tmp_path):
+    reqs = requests_for("A", [40, 9], 6)
+    steps = plans.unequal_batches([{rid: (toks, len(toks) - 4) for rid, toks in reqs.items()}])
+    out = str(tmp_path / "out")
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folders["A"], "--dtype", "float32",
+                           "--out", out, "--max-tokens", str(plans.max_live_tokens(steps))],
+                          input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+    got = plans.collect(steps, lambda i: np.fromfile(os.path.join(out, f"{i}.f32"), dtype="<f4"), Z_A["vocab"])
+    against_plain(folders["A"], got, reqs, "float32", "trace program")
+
+
+def test_a_sequence_cannot_outgrow_the_positions_the_model_has(folders):
+    from rust_inference_amd.errors import InferenceError
+    from rust_inference_amd.engine.step import Engine, StepEntry
+    model = loaded(folders, "C", "float32")
+    cache = model.new_cache(max_tokens=2048, num_slots=2, max_seq_len=2048)
+    assert cache.max_seq_len == Z_C["max_positions"]
+    engine = Engine(model, cache)
+    slot = cache.acquire()
+    with pytest.raises(InferenceError):
+        engine.step([StepEntry(slot, [1] * (Z_C["max_positions"] + 1), "last")])
+    cache.release(slot)
+    cache.check_consistent()
