@@ -110,7 +110,8 @@ int ri_relu_squared(void* out, const void* y, int dtype, long total, void* strea
 int ri_attention_prefill_bf16(void* out, const void* qkv, int q_stride, const void* k_pages, const void* v_pages,
                               const int32_t* cu_seqlens, const int32_t* tok_pos, const int32_t* page_table,
                               int table_width, int seqs, int max_new, int heads, int kv_heads, int head_dim,
-                              int page_size, int window, float scale, void* stream);
+                              int page_size, int window, float scale, float softcap, void* stream);
+// (softcap > 0, here and in the decode form: a score s becomes softcap * tanh(s / softcap) before the softmax)
 
 // Decode form: exactly one new token per sequence; keys in chunks of 256 (in a step of few workgroups each cut into
 // 2 or 4 pieces), joined by a second kernel.
@@ -126,7 +127,8 @@ int ri_attention_decode_streams(int seqs, int kv_heads, int max_chunks);
 int ri_attention_decode_bf16(void* out, float* workspace, const void* qkv, int q_stride, const void* k_pages,
                              const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
                              const int32_t* page_table, int table_width, int seqs, int max_chunks, int heads,
-                             int kv_heads, int head_dim, int page_size, int window, float scale, int tiled_out, void* stream);
+                             int kv_heads, int head_dim, int page_size, int window, float scale, float softcap,
+                             int tiled_out, void* stream);
 
 // tiled_out (both decode forms): the result [seqs, heads * head_dim] is written in the matrix cores' operand order
 // (see tiled_at in common.h) for the packed product that reads it.

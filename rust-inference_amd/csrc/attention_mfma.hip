@@ -115,7 +115,22 @@ struct Columns {
     floatx4 o[NT][DH / 16];
     float m[NT], l[NT];
     int qpos[NT], lo[NT];         // the column's query position (-1: no such column) and first visible key
+    // a cap c on the scores, s <- c tanh(s / c) with s = scale (q . k), applied to the raw products so that what
+    // follows still multiplies by the scale: (q . k) <- cap_post * tanh((q . k) * cap_pre), cap_pre = scale / c,
+    // cap_post = c / scale; both 0: no cap
+    float cap_pre, cap_post;
 };
+
+// tanh through one exponential: 1 - 2 / (e^(2x) + 1), exact at both ends (e^(2x) = inf or 0).
+__device__ __forceinline__ float tanh_by_exp(float x) {
+    const float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
+__device__ __forceinline__ void cap_scores(float (&s)[8], float cap_pre, float cap_post) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s[e] = cap_post * tanh_by_exp(s[e] * cap_pre);
+}
 
 // One page for NT tiles of columns, in two halves so that the key fragments and the value fragments
 // need not be in registers at the same time.  `open` says that every key of the page is visible to
@@ -137,6 +152,7 @@ __device__ __forceinline__ void scores_and_weights(Columns<DH, NT>& c, const Fra
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][ks].v, c.q[j][ks].v, s1, 0, 0, 0);
         }
         float s[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+        if (c.cap_pre != 0.f) cap_scores(s, c.cap_pre, c.cap_post);
         if (!open) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -202,6 +218,7 @@ __device__ __forceinline__ void init_columns(Columns<DH, NT>& c) {
         c.l[j] = 0.f;
         c.qpos[j] = -1;
         c.lo[j] = 0;
+        c.cap_pre = c.cap_post = 0.f;
 #pragma unroll
         for (int ks = 0; ks < DH / 32; ++ks) c.q[j][ks].u = make_uint4(0, 0, 0, 0);
 #pragma unroll
@@ -226,6 +243,7 @@ __device__ __forceinline__ void scores_of(const Columns<DH, NT>& c, const Frag (
             s[j][e] = s0[e];
             s[j][4 + e] = s1[e];
         }
+        if (c.cap_pre != 0.f) cap_scores(s[j], c.cap_pre, c.cap_post);
     }
 }
 
@@ -345,7 +363,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                          const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ tok_pos,
                          const int32_t* __restrict__ page_table, int table_width, int heads, int kv_heads,
-                         int window, float scale_log2) {
+                         int window, float scale_log2, float cap_pre, float cap_post) {
     __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][PAGE * LdsPage<DH>::KS];
     __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][DH * LdsPage<DH>::VS];
     const int lane = threadIdx.x & 63;
@@ -364,6 +382,8 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
 
     Columns<DH, NT> c;
     init_columns<DH, NT>(c);
+    c.cap_pre = cap_pre;
+    c.cap_post = cap_post;
     const int jg = lane >> 4;
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
@@ -508,7 +528,7 @@ __global__ void __launch_bounds__(CW * 64)
 attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, int q_stride,
                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
-                        int heads, int kv_heads, int window, float scale_log2, int max_chunks) {
+                        int heads, int kv_heads, int window, float scale_log2, int max_chunks, float cap_pre, float cap_post) {
     __shared__ float o_lds[CW][DH * 17];           // [d * 17 + col]: no bank conflicts either way
     __shared__ float ml_lds[CW][2][16];
     const int lane = threadIdx.x & 63;
@@ -530,6 +550,8 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
     const bool has = page * PAGE <= qpos && page * PAGE + PAGE - 1 >= lo;
     Columns<DH, 1> c;
     init_columns<DH, 1>(c);
+    c.cap_pre = cap_pre;
+    c.cap_post = cap_post;
     const int jg = lane >> 4, col = lane & 15;
     {
         const bf16_t* qp = qkv + (long)tok * q_stride + (kvh * group + min(col, group - 1)) * DH + jg * 8;
@@ -813,7 +835,7 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
                           const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
                           const float* __restrict__ inv_freq, bf16_t* k_pages, bf16_t* v_pages,
                           const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
-                          int heads, int kv_heads, int window, float scale_log2, int splits, int tiled) {
+                          int heads, int kv_heads, int window, float scale_log2, int splits, int tiled, float cap_pre, float cap_post) {
     static_assert(!FUSED || DH <= 128, "one (d, d + DH/2) pair per lane");
     __shared__ float o_lds[W][DH * 17];
     __shared__ float ml_lds[W][2][16];
@@ -864,6 +886,8 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
     // read that page, the last of the run, so nothing has to be patched into fragments afterwards.
     Columns<DH, 1> c;
     init_columns<DH, 1>(c);
+    c.cap_pre = cap_pre;
+    c.cap_post = cap_post;
     const int jg = lane >> 4, col = lane & 15;
     fetch_table(0);
     if (FUSED) {
@@ -1193,7 +1217,9 @@ extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_strid
                                          const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
                                          const int32_t* page_table, int table_width, int seqs, int max_new,
                                          int heads, int kv_heads, int head_dim, int page_size, int window,
-                                         float scale, void* stream) {
+                                         float scale, float softcap, void* stream) {
+    const float cap_pre = softcap > 0.f ? scale / softcap : 0.f, cap_post = softcap > 0.f ? softcap / scale : 0.f;
+    RI_REQUIRE(scale > 0.f, "attention_prefill_bf16: the scale %g must be positive", (double)scale);
     if (check_common("attention_prefill_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width)) return 1;
     const int group = heads / kv_heads;
     RI_REQUIRE(seqs > 0 && seqs <= 65535 && max_new > 0, "attention_prefill_bf16: seqs %d, max_new %d", seqs, max_new);
@@ -1210,7 +1236,8 @@ extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_strid
     case DH * 8 + NT:                                                                                            \
         attn_prefill_mfma_kernel<DH, NT><<<grid, 256, 0, s>>>(                                                   \
             (bf16_t*)out, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,          \
-            cu_seqlens, tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2);                  \
+            cu_seqlens, tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, cap_pre,          \
+            cap_post);                                                                                           \
         break;
     switch (head_dim * 8 + nt_tiles) {
         RI_PREFILL_CASE(32, 4)
@@ -1255,7 +1282,9 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
                                         const void* k_pages, const void* v_pages, const int32_t* cu_seqlens,
                                         const int32_t* tok_pos, const int32_t* page_table, int table_width, int seqs,
                                         int max_chunks, int heads, int kv_heads, int head_dim, int page_size,
-                                        int window, float scale, int tiled_out, void* stream) {
+                                        int window, float scale, float softcap, int tiled_out, void* stream) {
+    const float cap_pre = softcap > 0.f ? scale / softcap : 0.f, cap_post = softcap > 0.f ? softcap / scale : 0.f;
+    RI_REQUIRE(scale > 0.f, "attention_decode_bf16: the scale %g must be positive", (double)scale);
     if (check_common("attention_decode_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width)) return 1;
     RI_REQUIRE(!tiled_out || (seqs <= 64 && head_dim % 32 == 0), "attention_decode_bf16: tiled rows are at most 64 (%d)", seqs);
     const int group = heads / kv_heads;
@@ -1275,12 +1304,12 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
             attn_decode_stream_kernel<DH, false, 8><<<sgrid, 8 * 64, 0, s>>>(                                     \
                 (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, nullptr, nullptr, 0.f, nullptr,            \
                 (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
-                scale_log2, splits, tiled_out);                                                                   \
+                scale_log2, splits, tiled_out, cap_pre, cap_post);                                                \
         else                                                                                                      \
             attn_decode_stream_kernel<DH, false, 4><<<sgrid, 4 * 64, 0, s>>>(                                     \
                 (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, nullptr, nullptr, 0.f, nullptr,            \
                 (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
-                scale_log2, splits, tiled_out);                                                                   \
+                scale_log2, splits, tiled_out, cap_pre, cap_post);                                                \
         if (splits > 1) launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, -1, splits, tiled_out, s); \
         break;
         switch (head_dim) {
@@ -1298,7 +1327,7 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
     case DH * 16 + CW:                                                                                            \
         attn_decode_mfma_kernel<DH, CW><<<pgrid, CW * 64, 0, s>>>(                                                \
             workspace, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
-            tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, all);                          \
+            tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, all, cap_pre, cap_post);      \
         launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, all, tiled_out, s, CW * PAGE);     \
         break;
     switch (head_dim * 16 + DECODE_WAVES / pieces) {
@@ -1347,12 +1376,12 @@ extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const
             attn_decode_stream_kernel<DH, true, 8><<<sgrid, 8 * 64, 0, s>>>(                                      \
                 (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq,             \
                 (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
-                scale_log2, splits, tiled_out);                                                                   \
+                scale_log2, splits, tiled_out, 0.f, 0.f);                                                         \
         else                                                                                                      \
             attn_decode_stream_kernel<DH, true, 4><<<sgrid, 4 * 64, 0, s>>>(                                      \
                 (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq,             \
                 (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
-                scale_log2, splits, tiled_out);                                                                   \
+                scale_log2, splits, tiled_out, 0.f, 0.f);                                                         \
         if (splits > 1) launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, -1, splits, tiled_out, s); \
         break;
         switch (head_dim) {

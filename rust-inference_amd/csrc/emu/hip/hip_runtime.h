@@ -117,6 +117,7 @@ static inline typename std::common_type<A, B>::type max(A a, B b) {
     return (T)a < (T)b ? (T)b : (T)a;
 }
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
+#define __builtin_amdgcn_rcpf(x) (1.0f / (x))
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
 
 // ---- atomics: one host thread runs everything

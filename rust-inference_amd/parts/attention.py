@@ -216,8 +216,7 @@ class GroupedQueryAttention(Mixer):
                                         page_table, store.k_pages, store.v_pages, self.heads, self.kv_heads,
                                         self.head_dim, self.v_dim)
         with profiler.section(profiler.ATTENTION):
-            o = ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, self.heads,
-                              self.kv_heads, self.head_dim, self.window, self.scale, self.softcap)
+            o = self.attend(qkv, ctx, store, page_table)
         return self.project_out(o, link)
 
     def project_out(self, o, link):
@@ -231,19 +230,23 @@ class GroupedQueryAttention(Mixer):
         sequence, or any number), the generic kernel for everything else."""
         args = (self.heads, self.kv_heads, self.head_dim, self.window, self.scale)
         group = self.heads // self.kv_heads
+        cap = self.softcap
+        if self.v_dim != self.head_dim:          # value heads of their own size: the generic kernel alone takes them
+            return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args, cap)
         if self.rt.invariant:
             # one kernel for prompts and single tokens alike: in the prompt kernel a token's sums run over its
             # sequence's pages in order whatever the other rows of its tile are (a page that a row does not
             # see changes none of its bits); the generic kernel where that one does not take the sizes
             if ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, False):
                 return ops.attention_prefill_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
-                                                  page_table, ctx.B, ctx.max_new, *args)
-            return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args)
+                                                  page_table, ctx.B, ctx.max_new, *args, cap)
+            return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args, cap)
         if ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, ctx.is_decode):
             if ctx.is_decode:
                 return ops.attention_decode_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
                                                  page_table, ctx.B, ctx.max_len, *args,
-                                                 tiled_out=self.rt.takes_tiled(self.w_o, ctx.B, self.b_o is None))
+                                                 tiled_out=self.rt.takes_tiled(self.w_o, ctx.B, self.b_o is None),
+                                                 softcap=cap)
             return ops.attention_prefill_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
-                                              page_table, ctx.B, ctx.max_new, *args)
-        return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args)
+                                              page_table, ctx.B, ctx.max_new, *args, cap)
+        return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args, cap)

@@ -60,8 +60,8 @@ class GatedLinearAttention(Mixer):
             raise ConfigError(f"{n['a1']} has {weights[n['a1']].shape[0]} rows, {n['a2']} {weights[n['a2']].shape[1]} columns")
         fused = torch.cat([weights[n["q"]], weights[n["k"]], weights[n["v"]], weights[n["g"]]], 0)
         self.w_qkvg = rt.pack(rt.place_matrix(fused))
-        self.w_a1 = rt.place_matrix(weights[n["a1"]])
-        self.w_a2 = rt.place_matrix(weights[n["a2"]])
+        self.w_a1 = rt.pack(rt.place_matrix(weights[n["a1"]]))
+        self.w_a2 = rt.pack(rt.place_matrix(weights[n["a2"]]))
         self.z_bias = rt.place_gain(weights[n["a2_bias"]])
         self.gain = rt.place_gain(weights[n["norm"]])
         self.w_o = rt.pack(rt.place_matrix(weights[n["o"]]), parts_ok=True)
@@ -73,7 +73,7 @@ class GatedLinearAttention(Mixer):
         rt, hk, hv = self.rt, self.heads * self.dim, self.heads * self.vdim
         with profiler.section(profiler.QKV_PROJECTION):
             proj = ops.as_rows(rt.linear_packed(x, self.w_qkvg))          # [T, q | k | v | g]
-            z = rt.linear(rt.linear(x, self.w_a1), self.w_a2, out_dtype=torch.float32)
+            z = rt.linear_packed(ops.as_rows(rt.linear_packed(x, self.w_a1)), self.w_a2, out_dtype=torch.float32)
         with profiler.section(profiler.ATTENTION):
             o = ops.gla_scan(proj, 0, hk, 2 * hk, z, self.z_bias, self.tau, self.dim ** -0.5, store, ctx.cu_seqlens,
                              ctx.slots, self.heads, self.dim, self.vdim)

@@ -58,12 +58,13 @@ ONE_UNIT = ("one_run or mfma_prefill_attention or (mfma_attention_window_edges a
 PYTEST = ["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider"]
 KERNEL_TESTS, SMALL_MACHINE = os.path.join(HERE, "test_kernels_gpu.py"), os.path.join(HERE, "small_machine_kernels.py")
 SAMPLER_TESTS = os.path.join(HERE, "test_sampling_gpu.py")
+ZIDEPEL_TESTS = os.path.join(HERE, "test_zidepel_kernels_gpu.py")
 SAMPLER_SELECT = "(same_token_as_the_plain_sampler or top_p_drops) and not large"     # not the 151,936 entries, not the engine
 
 
 @pytest.fixture(scope="module")
 def runs():
-    """The four emulated runs, side by side (each is a pytest of its own; together they take what the longest takes)."""
+    """The emulated runs, side by side (each is a pytest of its own; together they take what the longest takes)."""
     from rust_inference_amd.errors import KernelError
     try:
         sys.path.insert(0, HERE)
@@ -76,6 +77,7 @@ def runs():
         "sixteen units": _start([*PYTEST, SMALL_MACHINE], {"RI_EMU_COMPUTE_UNITS": "16"}),
         "one unit": _start([*PYTEST, *_workers(2), SMALL_MACHINE, KERNEL_TESTS, "-k", ONE_UNIT], {"RI_EMU_COMPUTE_UNITS": "1"}),
         "sampler": _start([*PYTEST, *_workers(2), SAMPLER_TESTS, "-k", SAMPLER_SELECT]),
+        "zidepel": _start([*PYTEST, *_workers(2), ZIDEPEL_TESTS]),
     }
     done = {}
     try:
@@ -103,6 +105,13 @@ def test_the_kernel_tests_pass_on_the_cpu_build_between_guard_pages(runs):
 
 def test_the_sampler_tests_pass_on_the_cpu_build_between_guard_pages(runs):
     _passed(runs["sampler"], 33)
+
+
+def test_the_kernels_of_the_zidepel_design_pass_on_the_cpu_build_between_guard_pages(runs):
+    """tests/test_zidepel_kernels_gpu.py: residual streams and layer norm, the embedding with positions, norm,
+    temperature and cache write, capped attention (generic and on the emulated matrix cores), the gated linear
+    recurrence, the squared ReLU."""
+    _passed(runs["zidepel"])
 
 
 @pytest.mark.parametrize("units, tests", [("sixteen units", 7), ("one unit", 61)])

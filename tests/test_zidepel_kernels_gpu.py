@@ -218,6 +218,39 @@ def test_one_far_key_is_found_and_the_cap_holds_it_back(ops):
             assert np.abs(f64(got[-1]) - v[97, 0]).max() > 0.05
 
 
+@pytest.mark.parametrize("form", ["prefill", "decode"])
+@pytest.mark.parametrize("dh, heads, kv_heads, cap", [(64, 8, 2, 4.0), (128, 4, 1, 11.0), (32, 2, 2, 0.7), (64, 4, 4, None)])
+def test_the_matrix_core_kernels_cap_their_scores(ops, form, dh, heads, kv_heads, cap):
+    """bfloat16, heads of 32, 64 and 128: prompts of unequal lengths, and one new token each after them, with
+    scores large enough for the cap to bend most of them."""
+    rng = np.random.default_rng(dh)
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dh, "vdim": dh, "scale": 0.4, "softcap": cap, "q_temp": None}
+    lens = [75, 1, 40] if form == "prefill" else [300, 33, 64]
+    T = sum(lens)
+    q, k, v = rng.normal(size=(T, heads, dh)), rng.normal(size=(T, kv_heads, dh)), rng.normal(size=(T, kv_heads, dh))
+    qkv, kp, vp, tok_pos, tok_seq, table = paged(ops, m, q, k, v, lens, torch.bfloat16)
+    r = f64(qkv)
+    rq, rk, rv = (r[:, :heads * dh].reshape(T, heads, dh), r[:, heads * dh:(heads + kv_heads) * dh].reshape(T, kv_heads, dh),
+                  r[:, (heads + kv_heads) * dh:].reshape(T, kv_heads, dh))
+    ops.qk_norm_temper_kv_write(qkv, None, None, 1e-5, None, tok_pos, tok_seq, table, kp, vp, heads, kv_heads, dh, dh)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    want = np.concatenate([Z.attention_core(m, rq[a:b], rk[a:b], rv[a:b], np.arange(b - a)).reshape(b - a, -1)
+                           for a, b in zip(cu[:-1], cu[1:])])
+    if form == "prefill":
+        got = ops.attention_prefill_bf16(qkv, kp, vp, t(cu, torch.int32), tok_pos, table, len(lens), max(lens), heads,
+                                         kv_heads, dh, None, m["scale"], cap)
+        close(got, want, BF16_OUT, "prefill")
+    else:
+        last = cu[1:] - 1                                      # each sequence's last token as its one new token
+        rows = guarded(qkv[torch.tensor(last, dtype=torch.long)].clone())
+        got = ops.attention_decode_bf16(rows, kp, vp, t(np.arange(len(lens) + 1), torch.int32),
+                                        t([n - 1 for n in lens], torch.int32), table, len(lens), max(lens), heads, kv_heads,
+                                        dh, None, m["scale"], softcap=cap)
+        close(got, want[last], BF16_OUT, "decode")
+    same = ops.attention(qkv, kp, vp, tok_pos, tok_seq, table, heads, kv_heads, dh, None, m["scale"], cap)
+    close(same, want, BF16_OUT, "the generic kernel on the same pages")
+
+
 # ---------------------------------------------------------------- gated linear attention
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads, dk, dv, lens", [(3, 24, 40, [19, 1, 8]), (2, 72, 16, [5]), (1, 200, 17, [3, 2])])
