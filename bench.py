@@ -2,6 +2,7 @@
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--model 8b|0.6b|1.7b|4b|14b|32b]
+    python bench.py --design zidepel [--size 0.6b|8b] [--layers L]      # another workload: see design_comparison below
 
 The default run has the layer sizes of Qwen3-8B with random weights
 (N(0, 0.02), norm gains 1 + N(0, 0.1), seed 2), a batch of 8 and prompts of 2,048 tokens in a
@@ -87,12 +88,13 @@ class Bench:
         self.cfg["num_hidden_layers"] = self.layers
         self.cfg["max_position_embeddings"] = context
         self.context, self.graphs = context, graphs
+        self.vocab = self.cfg["vocab_size"]
         torch.manual_seed(self.seed)
         self.model = random_model(self.cfg, seed=self.seed, dtype=torch.bfloat16)
         self.gen = torch.Generator().manual_seed(self.seed)
 
     def prompts(self, batch, n, span=None):
-        torch, vocab = self.torch, self.cfg["vocab_size"]
+        torch, vocab = self.torch, self.vocab
         if span and batch > 1:                                    # unequal lengths, prefilled together
             lens = torch.randint(span[0], span[1] + 1, (batch,), generator=self.gen).tolist()
             return [torch.randint(0, vocab, (m,), generator=self.gen).tolist() for m in lens]
@@ -172,6 +174,65 @@ class Bench:
         self.torch.cuda.empty_cache()
 
 
+class ShapeBench(Bench):
+    """The same measurements for any configuration the registry knows."""
+
+    def __init__(self, name, cfg, vocab, seed, context, graphs=True):
+        import torch
+        from rust_inference_amd.parts import random_model
+        self.torch, self.name, self.cfg, self.seed, self.vocab = torch, name, cfg, seed, vocab
+        self.context, self.graphs = context, graphs
+        self.model = random_model(cfg, seed=seed, dtype=torch.bfloat16)
+        self.gen = torch.Generator().manual_seed(seed)
+
+    def measure(self, prompt, batches, steps, warmup):
+        out = {}
+        sec = self.prefill(prompt)
+        out["prefill"] = {"tokens": prompt, "ms": round(1e3 * sec, 2), "tok_s": round(prompt / sec, 1)}
+        for n in batches:
+            dt, _, launches = self.decode(n, steps, warmup, prompt // 2, count_launches=self.graphs)
+            out[f"decode_b{n}"] = {"ms": round(1e3 * dt / steps, 3), "tok_s": round(n * steps / dt, 1), "launches": launches}
+        return out
+
+
+def zidepel_like(q, layers, vocab, context):
+    """A Zidepel configuration with the layer sizes of a Qwen3 one: the same width, heads and head size; the
+    feed-forward half again as wide, so that its two matrices hold what the other's three do; every fourth layer
+    (the third of four) gated linear attention with as many heads, no feed-forward behind it; four residual streams."""
+    d, h, g, dh = q["hidden_size"], q["num_attention_heads"], q["num_key_value_heads"], q["head_dim"]
+    att = {"type": "attention", "mlp": {"kind": "dense", "ff": q["intermediate_size"] * 3 // 2},
+           "mixer": {"heads": h, "kv_heads": g, "dim": dh, "vdim": dh, "scale": dh ** -0.5, "softcap": 30.0,
+                     "q_temp": {"coef": 0.1, "every": 512}}}
+    rec = {"type": "gla", "mlp": None, "mixer": {"heads": h, "dim": dh, "vdim": dh, "tau": 16.0, "rank": 16}}
+    return {"architecture": "Zidepel", "vocab": vocab, "width": d, "max_positions": context, "norm": {"eps": 1e-5},
+            "streams": 4, "layers": [rec if i % 4 == 2 else att for i in range(layers)]}
+
+
+def design_comparison(args) -> int:
+    """`--design zidepel`: prefill and decode of a Zidepel model beside the Qwen3 model of the same layer sizes
+    (random weights, `--layers` layers each, default 8, and a vocabulary of 32,768 for both so that the layers and not
+    the output matrix are what is timed).  One JSON line; the default workload and its line are not touched."""
+    sizes = {"0.6b": QWEN3_0_6B, "8b": QWEN3_8B}
+    layers, vocab, context = args.layers or 8, 32768, args.context
+    out = {"metric": "prefill and decode of the Zidepel design beside Qwen3 at equal layer sizes", "unit": "tok/s",
+           "n_gpus": 1, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids", "layers": layers,
+           "vocab": vocab, "steps": args.steps, "warmup": args.warmup, "sizes": {}}
+    for size in ([args.size] if args.size else ["0.6b", "8b"]):
+        q = dict(sizes[size], num_hidden_layers=layers, vocab_size=vocab, max_position_embeddings=context,
+                 tie_word_embeddings=False)
+        pair = {}
+        for name, cfg in (("qwen3", q), ("zidepel", zidepel_like(q, layers, vocab, context))):
+            b = ShapeBench(f"{name} at Qwen3-{size} layer sizes", cfg, vocab, 11, context, not args.no_graphs)
+            pair[name] = b.measure(args.prompt, (1, 8, 32), args.steps, args.warmup)
+            b.close()
+        out["sizes"][size] = pair
+    z, q = out["sizes"][next(iter(out["sizes"]))]["zidepel"], out["sizes"][next(iter(out["sizes"]))]["qwen3"]
+    out["value"], out["higher_is_better"] = z["decode_b8"]["tok_s"], True
+    out["vs_qwen3_decode_b8"] = round(z["decode_b8"]["tok_s"] / q["decode_b8"]["tok_s"], 3)
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -187,10 +248,15 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the other models")
     ap.add_argument("--no-other-models", action="store_true", help="skip the Qwen3-0.6B and Qwen3-32B points")
     ap.add_argument("--no-graphs", action="store_true", help="launch every kernel of a decode step from the host")
+    ap.add_argument("--design", choices=["zidepel"], default=None,
+                    help="another workload: this design beside Qwen3 at equal layer sizes (prefill, decode at batch 1, 8, 32)")
+    ap.add_argument("--size", choices=["0.6b", "8b"], default=None, help="with --design: one of the two layer sizes only")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this library is single-GPU, --gpus {args.gpus} is not run")
         return 2
+    if args.design:
+        return design_comparison(args)
 
     from rust_inference_amd.cache import PAGE_SIZE
 
