@@ -61,8 +61,11 @@ int ri_attention(void* out, const void* q, int act_dtype, int q_stride, const vo
 // projection qkv: [tokens, heads * dim + kv_heads * dim + kv_heads * vdim].  Per-head RMS norm of q and k (gains
 // may be NULL), then q *= 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1) in place (temp_coef 0: none).
 // k_pages: [pages, kv_heads, page_size, dim]; v_pages: [pages, kv_heads, vdim, page_size].
+// cu_seqlens (int32 [seqs + 1], may be NULL), seqs and max_new (most new tokens of a sequence) let values be
+// written a page at a time.
 int ri_qk_norm_temper_kv_write(void* qkv, int act_dtype, const float* q_gain, const float* k_gain, float eps,
                                float temp_coef, int temp_every, const int32_t* tok_pos, const int32_t* tok_seq,
+                               const int32_t* cu_seqlens, int seqs, int max_new,
                                const int32_t* page_table, int table_width, void* k_pages, void* v_pages,
                                int cache_dtype, int tokens, int heads, int kv_heads, int dim, int vdim, int page_size,
                                void* stream);
@@ -91,10 +94,10 @@ int ri_embed_positions_norm(float* out, const void* table, const void* positions
 // with alpha = exp(log_sigmoid(z + bias) / tau):   S <- diag(alpha_t) S + k_t v_t^T,   o_t = S^T (q_t * q_scale).
 // state: float32 [slots, heads, dim, vdim], read at the sequence's slot before its first token of the step and
 // written back after its last.  cu_seqlens: [seqs + 1] over the flat tokens; slots: [seqs].  out: float32
-// [tokens, heads * vdim].
-int ri_gla_scan(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off, const float* z,
+// [tokens, heads * vdim].  With more tokens than sequences (a prompt) z is overwritten by the decays.
+int ri_gla_scan(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off, float* z,
                 const float* z_bias, float tau, float q_scale, float* state, const int32_t* cu_seqlens,
-                const int32_t* slots, int seqs, int heads, int dim, int vdim, void* stream);
+                const int32_t* slots, int seqs, int tokens, int heads, int dim, int vdim, void* stream);
 
 // out[t, h, :] = rms_norm(o[t, h, :]) * gain * silu(gate[t, h, :]): o float32 [tokens, heads * vdim]; gate read
 // from proj rows at column g_off; out of act_dtype [tokens, heads * vdim].

@@ -5,7 +5,9 @@
 //
 // The scan walks a sequence's tokens in order; what runs side by side is everything else: a workgroup owns one
 // (sequence, head) and GLA_COLS columns of the state, its 256 threads as 16 columns x 16 slices of rows, every
-// thread keeping its rows of its column in registers.  Tokens go through in blocks of nb: a block's q, k, alpha
+// thread keeping its rows of its column (slice r: rows r * rpt .. r * rpt + rpt - 1, rpt = ceil(dim / 16); read
+// from LDS 16 bytes at a time where rpt is a multiple of 4) in registers.  For prompts the decays are made by a
+// pass of their own over all tokens at once (gla_decay_kernel), so that no logarithm stands in the walk.  Tokens go through in blocks of nb: a block's q, k, alpha
 // and v are staged in LDS (two buffers), the next block's loads are asked for before the block in work is
 // computed and stored after it, so memory's latency is paid once a block and behind the arithmetic; the 16
 // slices' shares of o_t meet through a shuffle inside a wavefront and through LDS between the four wavefronts,
@@ -24,12 +26,20 @@ __device__ __forceinline__ float log_sigmoid(float z) {
     return fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
 }
 
-template <typename TA>
+// z <- exp(log_sigmoid(z + bias) / tau) in place, for all tokens at once.
+__global__ void gla_decay_kernel(float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau, long total,
+                                 int width) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    z[e] = expf(log_sigmoid(z[e] + (z_bias ? z_bias[e % width] : 0.f)) * inv_tau);
+}
+
+template <typename TA, bool V4>
 __global__ void __launch_bounds__(256)
 gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, int q_off, int k_off, int v_off,
                 const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau, float q_scale,
                 float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
-                int heads, int dim, int vdim, int nb) {
+                int heads, int dim, int vdim, int nb, int z_is_decay) {
     extern __shared__ float lds[];                           // two buffers of nb tokens: q, k, alpha (dim each), v (16)
     __shared__ float part[2][GLA_MAX_NB][4][GLA_COLS];       // the wavefronts' shares of o_t, two blocks in flight
     const int b = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * GLA_COLS;
@@ -40,13 +50,11 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
     if (t1 <= t0) return;
     const int stride = 3 * dim + GLA_COLS, per = nb * dim;
     float* S = state + (((size_t)slots[b] * heads + h) * dim) * vdim + col;
+    const int rpt = (dim + GLA_SLICES - 1) / GLA_SLICES, row0 = r * rpt;   // this thread's rows: row0 .. row0 + rpt - 1
+    const int rows_here = max(0, min(rpt, dim - row0));
     float s[GLA_MAX_ROWS];
 #pragma unroll
-    for (int j = 0; j < GLA_MAX_ROWS; ++j) {
-        const int i = r + j * GLA_SLICES;
-        s[j] = (live && i < dim) ? S[(size_t)i * vdim] : 0.f;
-    }
-    const int rows_here = (dim - r + GLA_SLICES - 1) / GLA_SLICES;          // rows r, r + 16, ... below dim
+    for (int j = 0; j < GLA_MAX_ROWS; ++j) s[j] = (live && j < rows_here) ? S[(size_t)(row0 + j) * vdim] : 0.f;
 
     // a block's inputs on their way: every load is issued whatever the indices are, from a token and a column
     // pulled back inside the data
@@ -75,7 +83,7 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
                 float* at = buf + (size_t)(e / dim) * stride;
                 at[i] = rq[j] * q_scale;
                 at[dim + i] = rk[j];
-                at[2 * dim + i] = expf(log_sigmoid(rz[j] + (z_bias ? z_bias[h * dim + i] : 0.f)) * inv_tau);
+                at[2 * dim + i] = z_is_decay ? rz[j] : expf(log_sigmoid(rz[j] + (z_bias ? z_bias[h * dim + i] : 0.f)) * inv_tau);
             }
         }
         if (tid < nb * GLA_COLS) buf[(size_t)(tid / GLA_COLS) * stride + 3 * dim + tid % GLA_COLS] = rv;
@@ -92,12 +100,28 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
             const float* at = buf + (size_t)n * stride;
             const float v = at[3 * dim + c];
             float o = 0.f;
+            if (V4) {                                        // rpt a multiple of 4 and every slice whole: 16 bytes a read
 #pragma unroll
-            for (int j = 0; j < GLA_MAX_ROWS; ++j) {
-                if (j < rows_here) {
-                    const int i = r + j * GLA_SLICES;
-                    s[j] = at[2 * dim + i] * s[j] + at[dim + i] * v;
-                    o += s[j] * at[i];
+                for (int j = 0; j < GLA_MAX_ROWS; j += 4) {
+                    if (j < rpt) {
+                        const float4 q4 = *reinterpret_cast<const float4*>(at + row0 + j);
+                        const float4 k4 = *reinterpret_cast<const float4*>(at + dim + row0 + j);
+                        const float4 a4 = *reinterpret_cast<const float4*>(at + 2 * dim + row0 + j);
+                        s[j] = a4.x * s[j] + k4.x * v;
+                        s[j + 1] = a4.y * s[j + 1] + k4.y * v;
+                        s[j + 2] = a4.z * s[j + 2] + k4.z * v;
+                        s[j + 3] = a4.w * s[j + 3] + k4.w * v;
+                        o += (s[j] * q4.x + s[j + 1] * q4.y) + (s[j + 2] * q4.z + s[j + 3] * q4.w);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < GLA_MAX_ROWS; ++j) {
+                    if (j < rows_here) {
+                        const int i = row0 + j;
+                        s[j] = at[2 * dim + i] * s[j] + at[dim + i] * v;
+                        o += s[j] * at[i];
+                    }
                 }
             }
             // lanes of a wavefront: 4 slices x 16 columns
@@ -116,17 +140,15 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
         }
     }
 #pragma unroll
-    for (int j = 0; j < GLA_MAX_ROWS; ++j) {
-        const int i = r + j * GLA_SLICES;
-        if (live && i < dim) S[(size_t)i * vdim] = s[j];
-    }
+    for (int j = 0; j < GLA_MAX_ROWS; ++j)
+        if (live && j < rows_here) S[(size_t)(row0 + j) * vdim] = s[j];
 }
 
 extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off,
-                           const float* z, const float* z_bias, float tau, float q_scale, float* state,
-                           const int32_t* cu_seqlens, const int32_t* slots, int seqs, int heads, int dim, int vdim,
-                           void* stream) {
-    RI_REQUIRE(seqs > 0 && heads > 0 && dim > 0 && vdim > 0, "gla_scan: %d sequences, %d heads of %d x %d", seqs, heads, dim, vdim);
+                           float* z, const float* z_bias, float tau, float q_scale, float* state,
+                           const int32_t* cu_seqlens, const int32_t* slots, int seqs, int tokens, int heads, int dim,
+                           int vdim, void* stream) {
+    RI_REQUIRE(seqs > 0 && tokens >= seqs && heads > 0 && dim > 0 && vdim > 0, "gla_scan: %d sequences, %d heads of %d x %d", seqs, heads, dim, vdim);
     RI_REQUIRE(dim <= GLA_SLICES * GLA_MAX_ROWS, "gla_scan: key heads of %d exceed the kernel's %d", dim, GLA_SLICES * GLA_MAX_ROWS);
     RI_REQUIRE(heads <= 65535 && seqs <= 65535, "gla_scan: %d heads of %d sequences exceed one launch", heads, seqs);
     RI_REQUIRE(tau > 0.f, "gla_scan: tau %g must be positive", (double)tau);
@@ -138,12 +160,21 @@ extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row,
     int nb = GLA_STAGE * 256 / dim;
     nb = nb > GLA_MAX_NB ? GLA_MAX_NB : nb;                  // dim <= 512: at least two tokens a block
     const size_t lds = (size_t)2 * nb * (3 * dim + GLA_COLS) * sizeof(float);
-    if (act_dtype == RI_F32)
-        gla_scan_kernel<float><<<grid, 256, lds, s>>>(out, (const float*)proj, row, q_off, k_off, v_off, z, z_bias,
-                                                      1.0f / tau, q_scale, state, cu_seqlens, slots, heads, dim, vdim, nb);
-    else
-        gla_scan_kernel<bf16_t><<<grid, 256, lds, s>>>(out, (const bf16_t*)proj, row, q_off, k_off, v_off, z, z_bias,
-                                                       1.0f / tau, q_scale, state, cu_seqlens, slots, heads, dim, vdim, nb);
+    // a prompt: the decays of all its tokens in one pass, in place of z, before the walk
+    int z_is_decay = 0;
+    if (tokens > seqs) {
+        const long total = (long)tokens * heads * dim;
+        RI_REQUIRE((total + 255) / 256 <= 2147483647L, "gla_scan: %ld decays exceed one launch", total);
+        gla_decay_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(z, z_bias, 1.0f / tau, total, heads * dim);
+        z_is_decay = 1;
+    }
+    const bool v4 = dim % (4 * GLA_SLICES) == 0;             // every slice has a multiple of 4 rows, 16-byte aligned in LDS
+#define RI_GLA_GO(T, V)                                                                                              \
+    gla_scan_kernel<T, V><<<grid, 256, lds, s>>>(out, (const T*)proj, row, q_off, k_off, v_off, z, z_bias, 1.0f / tau,   \
+                                                 q_scale, state, cu_seqlens, slots, heads, dim, vdim, nb, z_is_decay)
+    if (act_dtype == RI_F32) { if (v4) RI_GLA_GO(float, true); else RI_GLA_GO(float, false); }
+    else                     { if (v4) RI_GLA_GO(bf16_t, true); else RI_GLA_GO(bf16_t, false); }
+#undef RI_GLA_GO
     RI_LAUNCH_CHECK("gla_scan");
     return 0;
 }

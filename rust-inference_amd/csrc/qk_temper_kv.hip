@@ -7,7 +7,8 @@
 //   k:    into k_pages [pages][kv_heads][page_size][dim];
 //   v:    copied into v_pages [pages][kv_heads][vdim][page_size] (transposed inside a page).
 //
-// Norm, logarithm and factor are float32; a q or k element is rounded once.  One wavefront per (token, head).
+// Norm, logarithm and factor are float32; a q or k element is rounded once.  One wavefront per (token, head) in
+// the general kernel; prompts of head sizes that allow it go through the 16-byte kernels further down.
 #include "api.h"
 #include "common.h"
 
@@ -63,9 +64,167 @@ __global__ void qk_norm_temper_kv_write_kernel(
     }
 }
 
+// ------------------------------------------------------------------ prompts: 16 bytes a lane, values a page at a time
+// For steps with more than one new token a sequence and head sizes of 8 lanes' worth of eight elements or a
+// power-of-two fraction (dim 8, 16, ... 512): a lane takes eight consecutive elements of a q or k head, so dim / 8
+// lanes make a head and a wavefront works on 512 / dim heads at once, every load and store 16 bytes (32 for
+// float32); one workgroup a token.  Values are written by the page-wise kernel below.
+template <typename T> struct Eight;
+template <> struct Eight<float> {
+    __device__ static void load(const float* p, float* o) {
+        const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    }
+    __device__ static void store(float* p, const float* v) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+};
+template <> struct Eight<bf16_t> {
+    __device__ static void load(const bf16_t* p, float* o) {
+        const uint4 v = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[2 * i] = __uint_as_float(w[i] << 16);
+            o[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+        }
+    }
+    __device__ static void store(bf16_t* p, const float* v) {
+        *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]),
+                                                  pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
+    }
+};
+
+template <typename TA, typename TC>
+__global__ void __launch_bounds__(256)
+qk_norm_temper_k_write_vec_kernel(TA* __restrict__ qkv, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
+                                  float eps, float temp_coef, int temp_every, const int32_t* __restrict__ tok_pos,
+                                  const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ page_table,
+                                  int table_width, TC* __restrict__ k_pages, int heads, int kv_heads, int dim, int vdim,
+                                  int page_size) {
+    const int lane = threadIdx.x & (RI_WAVE - 1), wave = threadIdx.x / RI_WAVE;
+    const int t = blockIdx.x;
+    const int lanes_per_head = dim / 8;                      // a power of two, at most 64
+    const int heads_at_once = RI_WAVE / lanes_per_head;
+    const int pos = tok_pos[t];
+    const int page = page_table[(size_t)tok_seq[t] * table_width + pos / page_size];
+    const float temper = temp_coef != 0.f ? 1.0f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.0f) : 1.0f;
+    const int qk_heads = heads + kv_heads;
+    TA* row = qkv + (size_t)t * ((size_t)qk_heads * dim + (size_t)kv_heads * vdim);
+    const int sub = lane / lanes_per_head, piece = lane % lanes_per_head;
+    for (int h0 = wave * heads_at_once; h0 < qk_heads; h0 += 4 * heads_at_once) {
+        const int hh = h0 + sub;
+        if (hh >= qk_heads) continue;                        // lanes of a head stay together: the shuffles below are safe
+        TA* x = row + (size_t)hh * dim + piece * 8;
+        float a[8];
+        Eight<TA>::load(x, a);
+        const bool is_q = hh < heads;
+        const float* gain = is_q ? q_gain : k_gain;
+        if (gain) {
+            float ss = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += a[e] * a[e];
+            for (int m = lanes_per_head / 2; m > 0; m >>= 1) ss += __shfl_xor(ss, m, RI_WAVE);
+            const float f = 1.0f / sqrtf(ss / (float)dim + eps);
+            float g[8];
+            Eight<float>::load(gain + piece * 8, g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[e] = a[e] * f * g[e];
+        }
+        if (is_q) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[e] *= temper;
+            Eight<TA>::store(x, a);
+        } else {
+            Eight<TC>::store(k_pages + (((size_t)page * kv_heads + (hh - heads)) * page_size + pos % page_size) * dim + piece * 8, a);
+        }
+    }
+}
+
+// Values into their pages, a page at a time: one workgroup per (32 positions touched by this step, sequence, kv
+// head) reads the new tokens' value heads as rows, turns them through LDS and writes channel rows.
+#define QT_TOKENS 32
+template <typename TA, typename TC>
+__global__ void __launch_bounds__(256)
+values_to_pages_kernel(const TA* __restrict__ qkv, size_t row_len, size_t v_off, const int32_t* __restrict__ cu_seqlens,
+                       const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
+                       TC* __restrict__ v_pages, int kv_heads, int vdim, int page_size) {
+    extern __shared__ float tile[];                          // [QT_TOKENS][vdim + 1]
+    const int b = blockIdx.y, kvh = blockIdx.z;
+    const int t_begin = cu_seqlens[b], n = cu_seqlens[b + 1] - t_begin;
+    if (n <= 0) return;
+    const int start = tok_pos[t_begin];                      // the sequence's new tokens sit at start .. start + n - 1
+    const int first = (start / QT_TOKENS + blockIdx.x) * QT_TOKENS;
+    const int lo = max(first, start), hi = min(first + QT_TOKENS - 1, start + n - 1);
+    if (lo > hi) return;
+    const int stride = vdim + 1;
+    const TA* from = qkv + v_off + (size_t)kvh * vdim;
+    const bool whole = lo == first && hi == first + QT_TOKENS - 1;
+    if (sizeof(TA) == 2 && whole && vdim % 8 == 0 && (row_len % 8) == 0 && (v_off % 8) == 0) {
+        const int pieces = vdim / 8;
+        for (int e = threadIdx.x; e < QT_TOKENS * pieces; e += blockDim.x) {
+            const int tt = e / pieces, d = (e - tt * pieces) * 8;
+            float v[8];
+            Eight<TA>::load(from + (size_t)(t_begin + first - start + tt) * row_len + d, v);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) tile[tt * stride + d + j] = v[j];
+        }
+    } else {
+        for (int e = threadIdx.x; e < (hi - lo + 1) * vdim; e += blockDim.x) {
+            const int tt = e / vdim, d = e - tt * vdim;
+            tile[(lo - first + tt) * stride + d] = to_f32(from[(size_t)(t_begin + lo - start + tt) * row_len + d]);
+        }
+    }
+    __syncthreads();
+    const int page = page_table[(size_t)b * table_width + first / page_size];
+    TC* base = v_pages + ((size_t)page * kv_heads + kvh) * page_size * vdim + first % page_size;
+    if (whole && page_size % 8 == 0) {
+        for (int e = threadIdx.x; e < vdim * (QT_TOKENS / 8); e += blockDim.x) {
+            const int d = e / (QT_TOKENS / 8), t8 = (e - d * (QT_TOKENS / 8)) * 8;
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = tile[(t8 + j) * stride + d];
+            Eight<TC>::store(base + (size_t)d * page_size + t8, v);
+        }
+    } else {
+        for (int e = threadIdx.x; e < vdim * QT_TOKENS; e += blockDim.x) {
+            const int d = e / QT_TOKENS, tt = e - d * QT_TOKENS;
+            if (first + tt >= lo && first + tt <= hi) from_f32(base + (size_t)d * page_size + tt, tile[tt * stride + d]);
+        }
+    }
+}
+
+template <typename TA, typename TC>
+static void launch_qk_temper(void* qkv, const float* q_gain, const float* k_gain, float eps, float temp_coef, int temp_every,
+                             const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* cu_seqlens, int seqs, int max_new,
+                             const int32_t* page_table, int table_width, void* k_pages, void* v_pages, int tokens,
+                             int heads, int kv_heads, int dim, int vdim, int page_size, hipStream_t s) {
+    const int lph = dim / 8;
+    const size_t row_len = (size_t)(heads + kv_heads) * dim + (size_t)kv_heads * vdim;
+    const bool pieces_fit = dim % 8 == 0 && lph <= 64 && (lph & (lph - 1)) == 0 &&
+                            (sizeof(TA) == 2 ? (row_len % 8 == 0) : (row_len % 4 == 0));
+    if (cu_seqlens && max_new > 1 && pieces_fit && page_size % QT_TOKENS == 0 && seqs <= 65535 && kv_heads <= 65535 &&
+        (size_t)QT_TOKENS * (vdim + 1) * sizeof(float) <= 65536) {
+        qk_norm_temper_k_write_vec_kernel<TA, TC><<<tokens, 256, 0, s>>>(
+            (TA*)qkv, q_gain, k_gain, eps, temp_coef, temp_every, tok_pos, tok_seq, page_table, table_width, (TC*)k_pages,
+            heads, kv_heads, dim, vdim, page_size);
+        dim3 grid((max_new + QT_TOKENS - 2) / QT_TOKENS + 1, seqs, kv_heads);      // the 32-position pieces a sequence may touch
+        values_to_pages_kernel<TA, TC><<<grid, 256, QT_TOKENS * (vdim + 1) * sizeof(float), s>>>(
+            (const TA*)qkv, row_len, (size_t)(heads + kv_heads) * dim, cu_seqlens, tok_pos, page_table, table_width,
+            (TC*)v_pages, kv_heads, vdim, page_size);
+        return;
+    }
+    const long items = (long)tokens * (heads + 2 * kv_heads);
+    qk_norm_temper_kv_write_kernel<TA, TC><<<(unsigned)((items + 3) / 4), 256, 0, s>>>(
+        (TA*)qkv, q_gain, k_gain, eps, temp_coef, temp_every, tok_pos, tok_seq, page_table, table_width, (TC*)k_pages,
+        (TC*)v_pages, tokens, heads, kv_heads, dim, vdim, page_size);
+}
+
 extern "C" int ri_qk_norm_temper_kv_write(void* qkv, int act_dtype, const float* q_gain, const float* k_gain, float eps,
                                           float temp_coef, int temp_every, const int32_t* tok_pos,
-                                          const int32_t* tok_seq, const int32_t* page_table, int table_width,
+                                          const int32_t* tok_seq, const int32_t* cu_seqlens, int seqs, int max_new,
+                                          const int32_t* page_table, int table_width,
                                           void* k_pages, void* v_pages, int cache_dtype, int tokens, int heads,
                                           int kv_heads, int dim, int vdim, int page_size, void* stream) {
     RI_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0, "qk_norm_temper_kv_write: tokens %d, heads %d, kv heads %d", tokens,
@@ -80,15 +239,16 @@ extern "C" int ri_qk_norm_temper_kv_write(void* qkv, int act_dtype, const float*
     const long items = (long)tokens * (heads + 2 * kv_heads);
     const long blocks = (items + 3) / 4;
     RI_REQUIRE(blocks <= 2147483647L, "qk_norm_temper_kv_write: %ld heads exceed one launch", items);
+    RI_REQUIRE(!cu_seqlens || (seqs > 0 && max_new > 0), "qk_norm_temper_kv_write: seqs %d, max_new %d", seqs, max_new);
     hipStream_t s = (hipStream_t)stream;
     if (act_dtype == RI_F32)
-        qk_norm_temper_kv_write_kernel<float, float><<<(unsigned)blocks, 256, 0, s>>>(
-            (float*)qkv, q_gain, k_gain, eps, temp_coef, temp_every, tok_pos, tok_seq, page_table, table_width,
-            (float*)k_pages, (float*)v_pages, tokens, heads, kv_heads, dim, vdim, page_size);
+        launch_qk_temper<float, float>(qkv, q_gain, k_gain, eps, temp_coef, temp_every, tok_pos, tok_seq, cu_seqlens, seqs,
+                                       max_new, page_table, table_width, k_pages, v_pages, tokens, heads, kv_heads, dim,
+                                       vdim, page_size, s);
     else
-        qk_norm_temper_kv_write_kernel<bf16_t, bf16_t><<<(unsigned)blocks, 256, 0, s>>>(
-            (bf16_t*)qkv, q_gain, k_gain, eps, temp_coef, temp_every, tok_pos, tok_seq, page_table, table_width,
-            (bf16_t*)k_pages, (bf16_t*)v_pages, tokens, heads, kv_heads, dim, vdim, page_size);
+        launch_qk_temper<bf16_t, bf16_t>(qkv, q_gain, k_gain, eps, temp_coef, temp_every, tok_pos, tok_seq, cu_seqlens,
+                                         seqs, max_new, page_table, table_width, k_pages, v_pages, tokens, heads,
+                                         kv_heads, dim, vdim, page_size, s);
     RI_LAUNCH_CHECK("qk_norm_temper_kv_write");
     return 0;
 }

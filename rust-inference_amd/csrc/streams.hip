@@ -89,11 +89,170 @@ streams_read_norm_kernel(TO* __restrict__ out, float* dst, const float* src, lon
     }
 }
 
+// The same for rows of up to 8192 elements (a multiple of 4) and up to four streams: every thread asks for all
+// its 16-byte pieces of all streams and of the waiting output up front and keeps them in registers, so a row's
+// loads are in flight together and a step of one row is one trip to memory, not one per element.  Loads are
+// issued whatever the indices are, from a column pulled back inside the row.
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 ld4(const bf16_t* p) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xFFFF0000u), __uint_as_float(w.y << 16),
+                       __uint_as_float(w.y & 0xFFFF0000u));
+}
+__device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void st4(bf16_t* p, float4 v) {
+    uint2 w;
+    w.x = pack_bf16x2(v.x, v.y);
+    w.y = pack_bf16x2(v.z, v.w);
+    *reinterpret_cast<uint2*>(p) = w;
+}
+__device__ __forceinline__ float4 fma4(float a, float4 x, float4 acc) {
+    return make_float4(fmaf(a, x.x, acc.x), fmaf(a, x.y, acc.y), fmaf(a, x.z, acc.z), fmaf(a, x.w, acc.w));
+}
+
+template <typename TP, typename TO, int S, int VPT>
+__global__ void __launch_bounds__(256)
+streams_read_norm_vec_kernel(TO* __restrict__ out, float* dst, const float* src, long src_copy_stride,
+                             const TP* __restrict__ pending, int parts, size_t part_stride,
+                             const float* __restrict__ mix, const float* __restrict__ outw,
+                             const float* __restrict__ inw, const float* __restrict__ gain,
+                             const float* __restrict__ bias, float eps, int kind, const int32_t* __restrict__ rows,
+                             int dim) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.x;
+    const size_t at = rows ? (size_t)rows[row] : (size_t)row;
+    const bool store = rows == nullptr && (pending != nullptr || dst != src);
+    float cm[S][S], co[S], ci[S];
+#pragma unroll
+    for (int a = 0; a < S; ++a) {
+#pragma unroll
+        for (int b = 0; b < S; ++b) cm[a][b] = mix ? mix[a * S + b] : (a == b ? 1.f : 0.f);
+        co[a] = outw ? outw[a] : 1.f;
+        ci[a] = inw ? inw[a] : 1.f;
+    }
+    const float* xs = src + at * (src_copy_stride ? (size_t)S * dim : (size_t)dim);
+    float* xd = dst + at * (size_t)S * dim;
+    const TP* pend = pending ? pending + at * dim : nullptr;
+    float4 x[VPT][S], y[VPT];
+    int col[VPT];
+    bool ok[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = (threadIdx.x + i * 256) * 4;
+        ok[i] = c < dim;
+        col[i] = ok[i] ? c : 0;
+#pragma unroll
+        for (int s = 0; s < S; ++s) x[i][s] = ld4(xs + (size_t)s * src_copy_stride + col[i]);
+        y[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (pend) {
+        for (int p = 0; p < parts; ++p) {
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                const float4 v = ld4(pend + p * part_stride + col[i]);
+                y[i] = make_float4(y[i].x + v.x, y[i].y + v.y, y[i].z + v.z, y[i].w + v.w);
+            }
+        }
+    }
+    float4 u[VPT];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int t = 0; t < S; ++t) {
+            float4 nx = x[i][t];
+            if (pend) {
+                nx = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int s = 0; s < S; ++s) nx = fma4(cm[s][t], x[i][s], nx);
+                nx = fma4(co[t], y[i], nx);
+            }
+            if (store && ok[i]) st4(xd + (size_t)t * dim + col[i], nx);
+            r = fma4(ci[t], nx, r);
+        }
+        if (!ok[i]) r = make_float4(0.f, 0.f, 0.f, 0.f);
+        u[i] = r;
+        sum += kind == ST_NORM_RMS ? (r.x * r.x + r.y * r.y) + (r.z * r.z + r.w * r.w) : (r.x + r.y) + (r.z + r.w);
+    }
+    TO* o = out + (size_t)row * dim;
+    float mean = 0.f, inv = 1.f;
+    if (kind != ST_NORM_NONE) {
+        const float total = block_sum(sum, scratch);
+        if (kind == ST_NORM_RMS) {
+            inv = 1.0f / sqrtf(total / (float)dim + eps);
+        } else {
+            mean = total / (float)dim;
+            float dev = 0.f;
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                if (ok[i]) {
+                    const float a = u[i].x - mean, b = u[i].y - mean, c = u[i].z - mean, d = u[i].w - mean;
+                    dev += (a * a + b * b) + (c * c + d * d);
+                }
+            }
+            inv = 1.0f / sqrtf(block_sum(dev, scratch) / (float)dim + eps);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        if (!ok[i]) continue;
+        float4 v = u[i];
+        if (kind != ST_NORM_NONE) {
+            const float4 g = ld4(gain + col[i]);
+            v = make_float4((v.x - mean) * inv * g.x, (v.y - mean) * inv * g.y, (v.z - mean) * inv * g.z, (v.w - mean) * inv * g.w);
+            if (bias) {
+                const float4 b = ld4(bias + col[i]);
+                v = make_float4(v.x + b.x, v.y + b.y, v.z + b.z, v.w + b.w);
+            }
+        }
+        st4(o + col[i], v);
+    }
+}
+
+template <typename TP, typename TO, int S>
+static void launch_streams_vec(TO* out, float* dst, const float* src, long scs, const TP* pending, int parts, size_t ps,
+                               const float* mix, const float* outw, const float* inw, const float* gain,
+                               const float* bias, float eps, int kind, const int32_t* rows, int n_rows, int dim,
+                               hipStream_t s) {
+#define RI_STREAMS_VEC(VPT)                                                                                           \
+    streams_read_norm_vec_kernel<TP, TO, S, VPT><<<n_rows, 256, 0, s>>>(out, dst, src, scs, pending, parts, ps, mix, outw, \
+                                                                        inw, gain, bias, eps, kind, rows, dim)
+    if (dim <= 1024) RI_STREAMS_VEC(1);
+    else if (dim <= 2048) RI_STREAMS_VEC(2);
+    else if (dim <= 4096) RI_STREAMS_VEC(4);
+    else RI_STREAMS_VEC(8);
+#undef RI_STREAMS_VEC
+}
+
+template <typename TP, typename TO>
+static bool try_streams_vec(TO* out, float* dst, const float* src, long scs, int S, const TP* pending, int parts, size_t ps,
+                            const float* mix, const float* outw, const float* inw, const float* gain, const float* bias,
+                            float eps, int kind, const int32_t* rows, int n_rows, int dim, hipStream_t s) {
+    if (dim % 4 || dim > 8192 || S > 4) return false;
+#define RI_STREAMS_S(SS)                                                                                             \
+    case SS: launch_streams_vec<TP, TO, SS>(out, dst, src, scs, pending, parts, ps, mix, outw, inw, gain, bias, eps, kind, \
+                                            rows, n_rows, dim, s); break;
+    switch (S) {
+        RI_STREAMS_S(1)
+        RI_STREAMS_S(2)
+        RI_STREAMS_S(3)
+        RI_STREAMS_S(4)
+    }
+#undef RI_STREAMS_S
+    return true;
+}
+
 template <typename TP>
 static void launch_streams(void* out, int out_dtype, float* dst, const float* src, long scs, int S, const TP* pending,
                            int parts, size_t ps, const float* mix, const float* outw, const float* inw,
                            const float* gain, const float* bias, float eps, int kind, const int32_t* rows, int n_rows,
                            int dim, hipStream_t s) {
+    if (out_dtype == RI_F32 ? try_streams_vec<TP, float>((float*)out, dst, src, scs, S, pending, parts, ps, mix, outw, inw, gain,
+                                                          bias, eps, kind, rows, n_rows, dim, s)
+                            : try_streams_vec<TP, bf16_t>((bf16_t*)out, dst, src, scs, S, pending, parts, ps, mix, outw, inw,
+                                                           gain, bias, eps, kind, rows, n_rows, dim, s))
+        return;
     const size_t lds = (size_t)dim * sizeof(float);
     if (out_dtype == RI_F32)
         streams_read_norm_kernel<TP, float><<<n_rows, 256, lds, s>>>((float*)out, dst, src, scs, S, pending, parts, ps,

@@ -29,14 +29,14 @@ _SIGNATURES = {
     "ri_attention": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                      c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
     "ri_qk_norm_temper_kv_write": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_float, c_int, c_void_p, c_void_p,
-                                   c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                   c_void_p],
+                                   c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                                   c_int, c_int, c_int, c_int, c_void_p],
     "ri_streams_read_norm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p,
                              c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_int, c_int, c_void_p],
     "ri_embed_positions_norm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                 c_int, c_int, c_int, c_void_p],
     "ri_gla_scan": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float,
-                    c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                    c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gla_norm_gate": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_int, c_int, c_int,
                          c_void_p],
     "ri_relu_squared": [c_void_p, c_void_p, c_int, ctypes.c_long, c_void_p],
@@ -302,11 +302,13 @@ def attention(qkv, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, k
 
 
 def qk_norm_temper_kv_write(qkv, q_gain, k_gain, eps: float, temper, tok_pos, tok_seq, page_table, k_pages, v_pages,
-                            heads: int, kv_heads: int, dim: int, vdim: int) -> None:
+                            heads: int, kv_heads: int, dim: int, vdim: int, cu_seqlens=None, max_new: int = 0) -> None:
     """Per-head RMS norm of q and k (gains may be None), the query temperature ``temper = (coef, every)`` or None
     (``q *= 1 + coef * ln(floor((pos + 1) / every) + 1)``, q in place), k and v into their pages.
-    ``qkv: [T, heads * dim + kv_heads * dim + kv_heads * vdim]``."""
+    ``qkv: [T, heads * dim + kv_heads * dim + kv_heads * vdim]``.  With ``cu_seqlens`` (``[seqs + 1]``) and
+    ``max_new`` (the most new tokens of any sequence) a prompt's values go into their pages a page at a time."""
     tokens, stride = qkv.shape
+    seqs = cu_seqlens.shape[0] - 1 if cu_seqlens is not None else 0
     if stride != (heads + kv_heads) * dim + kv_heads * vdim:
         raise ShapeError(f"qkv rows of {stride} for {heads} + {kv_heads} heads of {dim} and {kv_heads} of {vdim}")
     pages, _, page_size, _ = k_pages.shape
@@ -314,6 +316,7 @@ def qk_norm_temper_kv_write(qkv, q_gain, k_gain, eps: float, temper, tok_pos, to
     _call("ri_qk_norm_temper_kv_write", _dev(qkv, "qkv"), code(qkv.dtype), _opt(q_gain, "q_gain", torch.float32, (dim,)),
           _opt(k_gain, "k_gain", torch.float32, (dim,)), float(eps), coef, every,
           _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+          _opt(cu_seqlens, "cu_seqlens", torch.int32), seqs, int(max_new),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1],
           _dev(k_pages, "k_pages", None, (pages, kv_heads, page_size, dim)),
           _dev(v_pages, "v_pages", k_pages.dtype, (pages, kv_heads, vdim, page_size)), code(k_pages.dtype),
@@ -374,7 +377,8 @@ def gla_scan(proj, q_off: int, k_off: int, v_off: int, z, z_bias, tau: float, q_
     """The gated linear recurrence over every sequence's new tokens; float32 ``[T, heads * vdim]``.
     ``proj: [T, row]`` holds q, k (``heads * dim``) and v (``heads * vdim``) at the given columns; ``z``
     (float32 ``[T, heads * dim]``) and ``z_bias`` give the decay ``exp(log_sigmoid(z + bias) / tau)``;
-    ``state: [slots, heads, dim, vdim]`` float32 is read and written at the sequences' slots."""
+    ``state: [slots, heads, dim, vdim]`` float32 is read and written at the sequences' slots.  In a step with more
+    tokens than sequences ``z`` is overwritten (by the decays, made for all tokens at once before the walk)."""
     tokens, row = proj.shape
     seqs = slots.shape[0]
     if state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, vdim):
@@ -384,7 +388,7 @@ def gla_scan(proj, q_off: int, k_off: int, v_off: int, z, z_bias, tau: float, q_
           _dev(z, "z", torch.float32, (tokens, heads * dim)), _opt(z_bias, "z_bias", torch.float32, (heads * dim,)),
           float(tau), float(q_scale), _dev(state, "state", torch.float32),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
-          seqs, heads, dim, vdim, _stream())
+          seqs, tokens, heads, dim, vdim, _stream())
     return out
 
 

@@ -214,7 +214,7 @@ class GroupedQueryAttention(Mixer):
         with profiler.section(profiler.QK_NORM_ROPE_APPEND):
             ops.qk_norm_temper_kv_write(qkv, self.q_gain, self.k_gain, self.eps, self.q_temper, ctx.tok_pos, ctx.tok_seq,
                                         page_table, store.k_pages, store.v_pages, self.heads, self.kv_heads,
-                                        self.head_dim, self.v_dim)
+                                        self.head_dim, self.v_dim, ctx.cu_seqlens, ctx.max_new)
         with profiler.section(profiler.ATTENTION):
             o = self.attend(qkv, ctx, store, page_table)
         return self.project_out(o, link)

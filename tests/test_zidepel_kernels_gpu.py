@@ -160,8 +160,10 @@ def paged(ops, m, q, k, v, lens, dtype, shuffle_seed=0):
     {"heads": 6, "kv_heads": 2, "dim": 24, "vdim": 40, "scale": 0.31, "softcap": 5.0, "q_temp": {"coef": 0.4, "every": 7}},
     {"heads": 3, "kv_heads": 3, "dim": 72, "vdim": 16, "scale": 0.05, "softcap": None, "q_temp": None},
     {"heads": 4, "kv_heads": 1, "dim": 16, "vdim": 16, "scale": 1.7, "softcap": 0.8, "q_temp": {"coef": 1.5, "every": 1}},
-], ids=["capped-tempered", "plain", "one-kv-head"])
-def test_norm_temperature_cache_write_and_capped_attention(ops, dtype, m):
+    {"heads": 4, "kv_heads": 2, "dim": 64, "vdim": 40, "scale": 0.2, "softcap": 9.0, "q_temp": {"coef": 0.3, "every": 16}},
+], ids=["capped-tempered", "plain", "one-kv-head", "heads-of-64"])
+@pytest.mark.parametrize("by_pages", [False, True], ids=["element-wise", "prompt-kernels"])
+def test_norm_temperature_cache_write_and_capped_attention(ops, dtype, m, by_pages):
     rng = np.random.default_rng(3)
     lens = [70, 1, 33]
     T = sum(lens)
@@ -172,7 +174,8 @@ def test_norm_temperature_cache_write_and_capped_attention(ops, dtype, m):
     rq, rk, rv = (f64(qkv)[:, :H * dk].reshape(T, H, dk), f64(qkv)[:, H * dk:(H + G) * dk].reshape(T, G, dk),
                   f64(qkv)[:, (H + G) * dk:].reshape(T, G, dv))
     temper = (m["q_temp"]["coef"], m["q_temp"]["every"]) if m["q_temp"] else None
-    ops.qk_norm_temper_kv_write(qkv, t(qg), t(kg), 1e-5, temper, tok_pos, tok_seq, table, kp, vp, H, G, dk, dv)
+    prompt = dict(cu_seqlens=t(np.concatenate([[0], np.cumsum(lens)]), torch.int32), max_new=max(lens)) if by_pages else {}
+    ops.qk_norm_temper_kv_write(qkv, t(qg), t(kg), 1e-5, temper, tok_pos, tok_seq, table, kp, vp, H, G, dk, dv, **prompt)
     got = ops.attention(qkv, kp, vp, tok_pos, tok_seq, table, H, G, dk, None, m["scale"], m["softcap"])
     want, want_q = [], []
     at = 0
@@ -187,7 +190,7 @@ def test_norm_temperature_cache_write_and_capped_attention(ops, dtype, m):
         want.append(Z.attention_core(m, qq, kk, rv[at:at + n], pos).reshape(n, -1))
         at += n
     tol = F32 * 4 if dtype == torch.float32 else BF16_OUT
-    close(qkv[:, :H * dk], np.concatenate(want_q).reshape(T, -1), 1e-6 if dtype == torch.float32 else 1e-9, "q in place")
+    close(qkv[:, :H * dk], np.concatenate(want_q).reshape(T, -1), 1e-6 if dtype == torch.float32 else 4e-3, "q in place")    # bfloat16: a last place where float32 and float64 round apart
     close(got, np.concatenate(want), tol, "attention")
 
 
@@ -253,7 +256,8 @@ def test_the_matrix_core_kernels_cap_their_scores(ops, form, dh, heads, kv_heads
 
 # ---------------------------------------------------------------- gated linear attention
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads, dk, dv, lens", [(3, 24, 40, [19, 1, 8]), (2, 72, 16, [5]), (1, 200, 17, [3, 2])])
+@pytest.mark.parametrize("heads, dk, dv, lens", [(3, 24, 40, [19, 1, 8]), (2, 72, 16, [5]), (1, 200, 17, [3, 2]),
+                                                  (2, 64, 32, [9, 2]), (1, 128, 16, [20, 1])])
 def test_gla_scan_and_output_gate(ops, dtype, heads, dk, dv, lens):
     rng = np.random.default_rng(dk)
     T = sum(lens)
@@ -287,6 +291,33 @@ def test_gla_scan_and_output_gate(ops, dtype, heads, dk, dv, lens):
     gate = p[:, g_off:g_off + heads * dv].reshape(T, heads, dv)
     want_out = Z.rms_norm(f64(o).reshape(T, heads, dv), gain, 1e-5) * Z.silu(gate)
     close(got, want_out.reshape(T, -1), F32 * 2 if dtype == torch.float32 else BF16_OUT, "normed and gated")
+
+
+def test_values_go_into_pages_from_any_start(ops):
+    """A prompt's portion that begins in the middle of a page and ends in the middle of another, beside a whole
+    page and a single token: the page-wise writer against the element-wise one."""
+    rng = np.random.default_rng(4)
+    H, G, dk, dv = 2, 2, 16, 24
+    starts, counts = [13, 64, 31], [70, 32, 1]
+    T = sum(counts)
+    width = 4
+    table = np.array([[5, 2, 9, 0], [7, 1, 3, 11], [4, 10, 6, 8]], dtype=np.int32)
+    tok_seq = np.concatenate([np.full(n, b) for b, n in enumerate(counts)]).astype(np.int32)
+    tok_pos = np.concatenate([np.arange(s, s + n) for s, n in zip(starts, counts)]).astype(np.int32)
+    cu = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    for dtype in (torch.bfloat16, torch.float32):
+        x = rng.normal(size=(T, (H + G) * dk + G * dv))
+        pages = []
+        for prompt in ({}, dict(cu_seqlens=t(cu, torch.int32), max_new=max(counts))):
+            qkv = t(x, dtype)
+            kp = guarded(torch.zeros((12, G, PAGE, dk), dtype=dtype, device=DEV))
+            vp = guarded(torch.zeros((12, G, dv, PAGE), dtype=dtype, device=DEV))
+            ops.qk_norm_temper_kv_write(qkv, t(np.ones(dk)), None, 1e-5, (0.5, 3), t(tok_pos, torch.int32), t(tok_seq, torch.int32),
+                                        t(table, torch.int32), kp, vp, H, G, dk, dv, **prompt)
+            pages.append((f64(qkv), f64(kp), f64(vp)))
+        for a, b in zip(pages[0][:2], pages[1][:2]):          # q and k: the two kernels sum a head's squares in another order
+            assert np.abs(a - b).max() <= (8e-3 if dtype == torch.bfloat16 else 1e-6) * np.abs(a).max()
+        assert np.array_equal(pages[0][2], pages[1][2]) and np.abs(pages[0][2]).sum() > 0          # values are copies
 
 
 def test_gla_token_by_token_is_the_scan(ops):
