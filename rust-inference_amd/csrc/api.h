@@ -104,6 +104,13 @@ int ri_gla_scan(float* out, const void* proj, int act_dtype, int row, int q_off,
 int ri_gla_norm_gate(void* out, const float* o, const void* proj, int act_dtype, int row, int g_off, const float* gain,
                      float eps, int tokens, int heads, int vdim, void* stream);
 
+// One new token a sequence (token b is sequence b's): the recurrence's step, the per-head RMS norm and the gate in
+// one kernel; out of act_dtype [seqs, heads * vdim].  ri_gla_step_fits: whether it takes these head sizes.
+int ri_gla_step_fits(int dim, int vdim);
+int ri_gla_step(void* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off, int g_off,
+                const float* z, const float* z_bias, float tau, float q_scale, float* state, const int32_t* slots,
+                const float* gain, float eps, int seqs, int heads, int dim, int vdim, void* stream);
+
 // out[i] = max(y[i], 0)^2.
 int ri_relu_squared(void* out, const void* y, int dtype, long total, void* stream);
 

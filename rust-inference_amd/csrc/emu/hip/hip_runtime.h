@@ -59,6 +59,8 @@ static inline hipError_t hipDeviceGetAttribute(int* value, hipDeviceAttribute_t,
 template <class T>
 static inline hipError_t hipGetSymbolAddress(void** p, T& symbol) { *p = (void*)&symbol; return hipSuccess; }
 static inline hipError_t hipMalloc(void**, size_t) { return hipErrorNoDevice; }
+enum hipFuncAttribute { hipFuncAttributeMaxDynamicSharedMemorySize = 8 };
+static inline hipError_t hipFuncSetAttribute(const void*, hipFuncAttribute, int) { return hipSuccess; }
 
 namespace emu {
 struct Thread {

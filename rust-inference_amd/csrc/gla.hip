@@ -18,8 +18,9 @@
 #define GLA_COLS 16
 #define GLA_SLICES 16
 #define GLA_MAX_ROWS 32          // rows of a column per thread: dim <= 16 * 32
-#define GLA_MAX_NB 8             // tokens of a block
-#define GLA_STAGE 4              // staged elements of q, k and z per thread and block: nb * dim <= 4 * 256
+#define GLA_MAX_NB 32            // tokens of a block
+#define GLA_STAGE 16             // staged elements of q, k and z per thread and block: nb * dim <= 16 * 256
+#define GLA_VSTAGE (GLA_MAX_NB * GLA_COLS / 256)
 
 __device__ __forceinline__ float log_sigmoid(float z) {
     // min(z, 0) - log(1 + exp(-|z|)): no overflow on either side
@@ -58,10 +59,11 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
 
     // a block's inputs on their way: every load is issued whatever the indices are, from a token and a column
     // pulled back inside the data
-    float rq[GLA_STAGE], rk[GLA_STAGE], rz[GLA_STAGE], rv;
+    float rq[GLA_STAGE], rk[GLA_STAGE], rz[GLA_STAGE], rv[GLA_VSTAGE];
     auto ask = [&](int tb) {
 #pragma unroll
         for (int j = 0; j < GLA_STAGE; ++j) {
+            if (j * 256 >= per) break;                       // (per is the same for all: no thread has an element here)
             const int e = min(tid + j * 256, per - 1);
             const int tok = min(tb + e / dim, t1 - 1), i = e % dim;
             const TA* x = proj + (size_t)tok * row;
@@ -69,15 +71,19 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
             rk[j] = to_f32(x[k_off + h * dim + i]);
             rz[j] = z[((size_t)tok * heads + h) * dim + i];
         }
-        const int e = min(tid, nb * GLA_COLS - 1);
-        const int tok = min(tb + e / GLA_COLS, t1 - 1), cc = min(col0 + e % GLA_COLS, vdim - 1);
-        rv = to_f32(proj[(size_t)tok * row + v_off + h * vdim + cc]);
+#pragma unroll
+        for (int j = 0; j < GLA_VSTAGE; ++j) {
+            const int e = min(tid + j * 256, nb * GLA_COLS - 1);
+            const int tok = min(tb + e / GLA_COLS, t1 - 1), cc = min(col0 + e % GLA_COLS, vdim - 1);
+            rv[j] = to_f32(proj[(size_t)tok * row + v_off + h * vdim + cc]);
+        }
     };
     auto put = [&](int which) {
         float* buf = lds + (size_t)which * nb * stride;
 #pragma unroll
         for (int j = 0; j < GLA_STAGE; ++j) {
             const int e = tid + j * 256;
+            if (j * 256 >= per) break;
             if (e < per) {
                 const int i = e % dim;
                 float* at = buf + (size_t)(e / dim) * stride;
@@ -86,14 +92,19 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
                 at[2 * dim + i] = z_is_decay ? rz[j] : expf(log_sigmoid(rz[j] + (z_bias ? z_bias[h * dim + i] : 0.f)) * inv_tau);
             }
         }
-        if (tid < nb * GLA_COLS) buf[(size_t)(tid / GLA_COLS) * stride + 3 * dim + tid % GLA_COLS] = rv;
+#pragma unroll
+        for (int j = 0; j < GLA_VSTAGE; ++j) {
+            const int e = tid + j * 256;
+            if (e < nb * GLA_COLS) buf[(size_t)(e / GLA_COLS) * stride + 3 * dim + e % GLA_COLS] = rv[j];
+        }
     };
     ask(t0);
     put(0);
     __syncthreads();
     int blk = 0;
     for (int tb = t0; tb < t1; tb += nb, ++blk) {
-        ask(tb + nb);
+        const bool more = tb + nb < t1;                      // the same for the whole workgroup
+        if (more) ask(tb + nb);
         const float* buf = lds + (size_t)(blk & 1) * nb * stride;
         for (int n = 0; n < nb; ++n) {
             if (tb + n >= t1) break;                         // the same for the whole workgroup
@@ -129,10 +140,10 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
             o += __shfl_xor(o, 32, RI_WAVE);
             if ((tid & (RI_WAVE - 1)) < GLA_COLS) part[blk & 1][n][wave][c] = o;
         }
-        put((blk + 1) & 1);
+        if (more) put((blk + 1) & 1);
         __syncthreads();
-        if (tid < nb * GLA_COLS) {
-            const int n = tid / GLA_COLS, cc = tid % GLA_COLS;
+        for (int e = tid; e < nb * GLA_COLS; e += 256) {
+            const int n = e / GLA_COLS, cc = e % GLA_COLS;
             if (tb + n < t1 && col0 + cc < vdim) {
                 const float (*p)[GLA_COLS] = part[blk & 1][n];
                 out[((size_t)(tb + n) * heads + h) * vdim + col0 + cc] = ((p[0][cc] + p[1][cc]) + p[2][cc]) + p[3][cc];
@@ -157,8 +168,12 @@ extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row,
     RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "gla_scan: dtype %d", act_dtype);
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((vdim + GLA_COLS - 1) / GLA_COLS, heads, seqs);
+    // tokens a block: as many as the staging registers hold (dim <= 512: at least eight), at most 32; 16 where
+    // the workgroups outnumber the compute units, so that several fit one unit's LDS; a step of single tokens 1
     int nb = GLA_STAGE * 256 / dim;
-    nb = nb > GLA_MAX_NB ? GLA_MAX_NB : nb;                  // dim <= 512: at least two tokens a block
+    nb = nb > GLA_MAX_NB ? GLA_MAX_NB : nb;
+    if (nb > 16 && (long)grid.x * grid.y * grid.z > ri_compute_units()) nb = 16;
+    if (tokens == seqs) nb = 1;
     const size_t lds = (size_t)2 * nb * (3 * dim + GLA_COLS) * sizeof(float);
     // a prompt: the decays of all its tokens in one pass, in place of z, before the walk
     int z_is_decay = 0;
@@ -169,11 +184,21 @@ extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row,
         z_is_decay = 1;
     }
     const bool v4 = dim % (4 * GLA_SLICES) == 0;             // every slice has a multiple of 4 rows, 16-byte aligned in LDS
+    // (more than 64 KB of dynamic LDS has to be asked for, once for every form of the kernel)
 #define RI_GLA_GO(T, V)                                                                                              \
+    if (lds > 48 * 1024) {                                                                                           \
+        static bool asked = false;                                                                                   \
+        if (!asked) {                                                                                                \
+            hipError_t e_ = hipFuncSetAttribute((const void*)gla_scan_kernel<T, V>,                                  \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);             \
+            RI_REQUIRE(e_ == hipSuccess, "gla_scan: %s", hipGetErrorString(e_));                                     \
+            asked = true;                                                                                            \
+        }                                                                                                            \
+    }                                                                                                                \
     gla_scan_kernel<T, V><<<grid, 256, lds, s>>>(out, (const T*)proj, row, q_off, k_off, v_off, z, z_bias, 1.0f / tau,   \
                                                  q_scale, state, cu_seqlens, slots, heads, dim, vdim, nb, z_is_decay)
-    if (act_dtype == RI_F32) { if (v4) RI_GLA_GO(float, true); else RI_GLA_GO(float, false); }
-    else                     { if (v4) RI_GLA_GO(bf16_t, true); else RI_GLA_GO(bf16_t, false); }
+    if (act_dtype == RI_F32) { if (v4) { RI_GLA_GO(float, true); } else { RI_GLA_GO(float, false); } }
+    else                     { if (v4) { RI_GLA_GO(bf16_t, true); } else { RI_GLA_GO(bf16_t, false); } }
 #undef RI_GLA_GO
     RI_LAUNCH_CHECK("gla_scan");
     return 0;
@@ -212,6 +237,58 @@ __global__ void gla_norm_gate_kernel(TA* __restrict__ out, const float* __restri
     }
 }
 
+// The same 16 bytes a lane, for value heads of 8 lanes' worth of eight elements or a power-of-two fraction (vdim 8,
+// 16, ... 512): vdim / 8 lanes make a head, a wavefront works on 512 / vdim heads at once.
+template <typename TA>
+__global__ void __launch_bounds__(256)
+gla_norm_gate_vec_kernel(TA* __restrict__ out, const float* __restrict__ o, const TA* __restrict__ proj, int row, int g_off,
+                         const float* __restrict__ gain, float eps, long items, int heads, int vdim) {
+    const int lanes_per_head = vdim / 8;
+    const int heads_at_once = RI_WAVE / lanes_per_head;
+    const int lane = threadIdx.x & (RI_WAVE - 1);
+    const long wave_id = (long)blockIdx.x * (blockDim.x / RI_WAVE) + threadIdx.x / RI_WAVE;
+    const long item = wave_id * heads_at_once + lane / lanes_per_head;
+    const int piece = lane % lanes_per_head;
+    if (item >= items) return;                               // lanes of a head leave together
+    const long t = item / heads;
+    const int h = (int)(item % heads);
+    const float* x = o + (size_t)item * vdim + piece * 8;
+    const float4 a = *reinterpret_cast<const float4*>(x), b = *reinterpret_cast<const float4*>(x + 4);
+    float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    float gate[8];
+    const TA* g = proj + (size_t)t * row + g_off + (size_t)h * vdim + piece * 8;
+    if (sizeof(TA) == 2) {
+        const uint4 w = *reinterpret_cast<const uint4*>(g);
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            gate[2 * i] = __uint_as_float(ww[i] << 16);
+            gate[2 * i + 1] = __uint_as_float(ww[i] & 0xFFFF0000u);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) gate[i] = to_f32(g[i]);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
+    for (int m = lanes_per_head / 2; m > 0; m >>= 1) ss += __shfl_xor(ss, m, RI_WAVE);
+    const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+    const float4 ga = *reinterpret_cast<const float4*>(gain + piece * 8), gb = *reinterpret_cast<const float4*>(gain + piece * 8 + 4);
+    const float gn[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
+    float r[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = v[e] * inv * gn[e] * (gate[e] / (1.0f + expf(-gate[e])));
+    TA* dst = out + (size_t)item * vdim + piece * 8;
+    if (sizeof(TA) == 2) {
+        *reinterpret_cast<uint4*>(dst) = make_uint4(pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3]), pack_bf16x2(r[4], r[5]),
+                                                    pack_bf16x2(r[6], r[7]));
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) from_f32(dst + e, r[e]);
+    }
+}
+
 extern "C" int ri_gla_norm_gate(void* out, const float* o, const void* proj, int act_dtype, int row, int g_off,
                                 const float* gain, float eps, int tokens, int heads, int vdim, void* stream) {
     RI_REQUIRE(tokens > 0 && heads > 0 && vdim > 0 && vdim <= RI_WAVE * GLA_NORM_PER_LANE,
@@ -222,6 +299,18 @@ extern "C" int ri_gla_norm_gate(void* out, const float* o, const void* proj, int
     const long blocks = (items + 3) / 4;
     RI_REQUIRE(blocks <= 2147483647L, "gla_norm_gate: %ld heads exceed one launch", items);
     hipStream_t s = (hipStream_t)stream;
+    const int lph = vdim / 8;
+    if (vdim % 8 == 0 && lph <= 64 && (lph & (lph - 1)) == 0 && row % 8 == 0 && g_off % 8 == 0) {
+        const long waves = (items + (64 / lph) - 1) / (64 / lph), vblocks = (waves + 3) / 4;
+        if (act_dtype == RI_F32)
+            gla_norm_gate_vec_kernel<float><<<(unsigned)vblocks, 256, 0, s>>>((float*)out, o, (const float*)proj, row, g_off,
+                                                                              gain, eps, items, heads, vdim);
+        else
+            gla_norm_gate_vec_kernel<bf16_t><<<(unsigned)vblocks, 256, 0, s>>>((bf16_t*)out, o, (const bf16_t*)proj, row,
+                                                                               g_off, gain, eps, items, heads, vdim);
+        RI_LAUNCH_CHECK("gla_norm_gate");
+        return 0;
+    }
     if (act_dtype == RI_F32)
         gla_norm_gate_kernel<float><<<(unsigned)blocks, 256, 0, s>>>((float*)out, o, (const float*)proj, row, g_off, gain, eps,
                                                                      items, heads, vdim);
@@ -229,5 +318,112 @@ extern "C" int ri_gla_norm_gate(void* out, const float* o, const void* proj, int
         gla_norm_gate_kernel<bf16_t><<<(unsigned)blocks, 256, 0, s>>>((bf16_t*)out, o, (const bf16_t*)proj, row, g_off, gain,
                                                                       eps, items, heads, vdim);
     RI_LAUNCH_CHECK("gla_norm_gate");
+    return 0;
+}
+
+// ------------------------------------------------------------------ one new token a sequence
+// The recurrence's step, the norm and the gate in one kernel: a workgroup owns one (sequence, head) and the whole
+// state of it, vdim / 4 groups of four columns x 256 / (vdim / 4) slices of rows, every thread's piece of the
+// state asked for up front in 16-byte loads (a step's time is the state's trip from memory and back), updated
+// in registers and stored; the slices' shares of o meet in LDS, where the head is normed and gated.
+#define GLA_STEP_ROWS 32
+
+template <typename TA, int ROWS>
+__global__ void __launch_bounds__(256)
+gla_step_kernel(TA* __restrict__ out, const TA* __restrict__ proj, int row, int q_off, int k_off, int v_off, int g_off,
+                const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau, float q_scale,
+                float* __restrict__ state, const int32_t* __restrict__ slots, const float* __restrict__ gain, float eps,
+                int heads, int dim, int vdim, int groups, int slices) {
+    __shared__ float qs[GLA_SLICES * GLA_MAX_ROWS], ks[GLA_SLICES * GLA_MAX_ROWS], as[GLA_SLICES * GLA_MAX_ROWS];
+    __shared__ __attribute__((aligned(16))) float red[1024];                 // [slices][vdim]
+    __shared__ float scratch[16];
+    const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int g = tid % groups, r = tid / groups;
+    const int rpt = (dim + slices - 1) / slices, row0 = r * rpt;
+    const int rows_here = r < slices ? max(0, min(rpt, dim - row0)) : 0;
+    float* S = state + (((size_t)slots[b] * heads + h) * dim) * vdim + 4 * g;
+    float4 s[ROWS];                                         // ROWS: 8, 16 or 32, the least that holds a slice
+#pragma unroll
+    for (int j = 0; j < ROWS; ++j)                           // every load issued, from a row pulled back inside the state
+        s[j] = *reinterpret_cast<const float4*>(S + (size_t)min(row0 + j, dim - 1) * vdim);
+    const TA* x = proj + (size_t)b * row;
+    for (int i = tid; i < dim; i += 256) {
+        qs[i] = to_f32(x[q_off + h * dim + i]) * q_scale;
+        ks[i] = to_f32(x[k_off + h * dim + i]);
+        as[i] = expf(log_sigmoid(z[((size_t)b * heads + h) * dim + i] + (z_bias ? z_bias[h * dim + i] : 0.f)) * inv_tau);
+    }
+    const TA* vx = x + v_off + h * vdim + 4 * g;
+    const float4 v = make_float4(to_f32(vx[0]), to_f32(vx[1]), to_f32(vx[2]), to_f32(vx[3]));
+    __syncthreads();
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int j = 0; j < ROWS; ++j) {
+        if (j < rows_here) {
+            const int i = row0 + j;
+            const float a = as[i], k = ks[i], q = qs[i];
+            s[j] = make_float4(a * s[j].x + k * v.x, a * s[j].y + k * v.y, a * s[j].z + k * v.z, a * s[j].w + k * v.w);
+            o = make_float4(o.x + s[j].x * q, o.y + s[j].y * q, o.z + s[j].z * q, o.w + s[j].w * q);
+            *reinterpret_cast<float4*>(S + (size_t)i * vdim) = s[j];
+        }
+    }
+    if (r < slices) *reinterpret_cast<float4*>(red + r * vdim + 4 * g) = o;
+    __syncthreads();
+    float mine[2] = {0.f, 0.f};
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+        const int c = tid + e * 256;
+        if (c < vdim) {
+            float t = 0.f;
+            for (int rr = 0; rr < slices; ++rr) t += red[rr * vdim + c];
+            mine[e] = t;
+            ss += t * t;
+        }
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)vdim + eps);
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+        const int c = tid + e * 256;
+        if (c < vdim) {
+            const float gate = to_f32(x[g_off + h * vdim + c]);
+            from_f32(out + ((size_t)b * heads + h) * vdim + c, mine[e] * inv * gain[c] * (gate / (1.0f + expf(-gate))));
+        }
+    }
+}
+
+// Whether the step kernel takes these head sizes: 1 yes, 0 no (then ri_gla_scan and ri_gla_norm_gate do).
+extern "C" int ri_gla_step_fits(int dim, int vdim) {
+    if (dim < 1 || dim > GLA_SLICES * GLA_MAX_ROWS || vdim < 4 || vdim % 4 || vdim > 512) return 0;
+    const int groups = vdim / 4, slices = 256 / groups;
+    return slices >= 1 && (dim + slices - 1) / slices <= GLA_STEP_ROWS && slices * vdim <= 1024;
+}
+
+extern "C" int ri_gla_step(void* out, const void* proj, int act_dtype, int row, int q_off, int k_off, int v_off, int g_off,
+                           const float* z, const float* z_bias, float tau, float q_scale, float* state,
+                           const int32_t* slots, const float* gain, float eps, int seqs, int heads, int dim, int vdim,
+                           void* stream) {
+    RI_REQUIRE(seqs > 0 && heads > 0 && ri_gla_step_fits(dim, vdim), "gla_step: %d sequences, %d heads of %d x %d", seqs,
+               heads, dim, vdim);
+    RI_REQUIRE(heads <= 65535 && seqs <= 65535, "gla_step: %d heads of %d sequences exceed one launch", heads, seqs);
+    RI_REQUIRE(tau > 0.f, "gla_step: tau %g must be positive", (double)tau);
+    RI_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && g_off >= 0 && q_off + heads * dim <= row && k_off + heads * dim <= row &&
+               v_off + heads * vdim <= row && g_off + heads * vdim <= row,
+               "gla_step: q, k, v, g at %d, %d, %d, %d do not fit rows of %d", q_off, k_off, v_off, g_off, row);
+    RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "gla_step: dtype %d", act_dtype);
+    hipStream_t s = (hipStream_t)stream;
+    const int groups = vdim / 4, slices = 256 / groups;
+    const dim3 grid(heads, seqs);
+    const int rpt = (dim + slices - 1) / slices;
+#define RI_STEP_GO(T, ROWS)                                                                                          \
+    gla_step_kernel<T, ROWS><<<grid, 256, 0, s>>>((T*)out, (const T*)proj, row, q_off, k_off, v_off, g_off, z, z_bias,   \
+                                                  1.0f / tau, q_scale, state, slots, gain, eps, heads, dim, vdim, groups, \
+                                                  slices)
+    if (act_dtype == RI_F32) {
+        if (rpt <= 8) RI_STEP_GO(float, 8); else if (rpt <= 16) RI_STEP_GO(float, 16); else RI_STEP_GO(float, 32);
+    } else {
+        if (rpt <= 8) RI_STEP_GO(bf16_t, 8); else if (rpt <= 16) RI_STEP_GO(bf16_t, 16); else RI_STEP_GO(bf16_t, 32);
+    }
+#undef RI_STEP_GO
+    RI_LAUNCH_CHECK("gla_step");
     return 0;
 }

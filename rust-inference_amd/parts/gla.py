@@ -59,7 +59,7 @@ class GatedLinearAttention(Mixer):
         if weights[n["a1"]].shape[0] != weights[n["a2"]].shape[1]:
             raise ConfigError(f"{n['a1']} has {weights[n['a1']].shape[0]} rows, {n['a2']} {weights[n['a2']].shape[1]} columns")
         fused = torch.cat([weights[n["q"]], weights[n["k"]], weights[n["v"]], weights[n["g"]]], 0)
-        self.w_qkvg = rt.pack(rt.place_matrix(fused))
+        self.w_qkvg = rt.pack(rt.place_matrix(fused), always=True)      # four projections in one: always worth its packed copy
         self.w_a1 = rt.pack(rt.place_matrix(weights[n["a1"]]))
         self.w_a2 = rt.pack(rt.place_matrix(weights[n["a2"]]))
         self.z_bias = rt.place_gain(weights[n["a2_bias"]])
@@ -74,6 +74,13 @@ class GatedLinearAttention(Mixer):
         with profiler.section(profiler.QKV_PROJECTION):
             proj = ops.as_rows(rt.linear_packed(x, self.w_qkvg))          # [T, q | k | v | g]
             z = rt.linear_packed(ops.as_rows(rt.linear_packed(x, self.w_a1)), self.w_a2, out_dtype=torch.float32)
+        if ctx.is_decode and ops.gla_step_fits(self.dim, self.vdim):
+            # one token a sequence: the step on the state, the norm and the gate are one kernel
+            with profiler.section(profiler.ATTENTION):
+                y = ops.gla_step(proj, 0, hk, 2 * hk, 2 * hk + hv, z, self.z_bias, self.tau, self.dim ** -0.5, store,
+                                 ctx.slots, self.gain, self.eps, self.heads, self.dim, self.vdim)
+            with profiler.section(profiler.OUT_PROJECTION):
+                return rt.linear_packed(y, self.w_o, parts_ok=True)
         with profiler.section(profiler.ATTENTION):
             o = ops.gla_scan(proj, 0, hk, 2 * hk, z, self.z_bias, self.tau, self.dim ** -0.5, store, ctx.cu_seqlens,
                              ctx.slots, self.heads, self.dim, self.vdim)

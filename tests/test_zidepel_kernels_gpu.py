@@ -262,8 +262,9 @@ def test_gla_scan_and_output_gate(ops, dtype, heads, dk, dv, lens):
     rng = np.random.default_rng(dk)
     T = sum(lens)
     tau = 3.5
-    proj = t(rng.normal(size=(T, 2 * heads * dk + 2 * heads * dv + 5)), dtype)      # q | k | 5 unused | v | g
-    q_off, k_off, v_off = 0, heads * dk, 2 * heads * dk + 5
+    pad = 8 if dk % 64 == 0 else 5                       # (rows of whole 16-byte pieces take the 16-byte norm and gate)
+    proj = t(rng.normal(size=(T, 2 * heads * dk + 2 * heads * dv + pad)), dtype)      # q | k | unused | v | g
+    q_off, k_off, v_off = 0, heads * dk, 2 * heads * dk + pad
     g_off = v_off + heads * dv
     z = rng.normal(size=(T, heads * dk)) * 3
     zb = rng.normal(size=heads * dk)
@@ -318,6 +319,40 @@ def test_values_go_into_pages_from_any_start(ops):
         for a, b in zip(pages[0][:2], pages[1][:2]):          # q and k: the two kernels sum a head's squares in another order
             assert np.abs(a - b).max() <= (8e-3 if dtype == torch.bfloat16 else 1e-6) * np.abs(a).max()
         assert np.array_equal(pages[0][2], pages[1][2]) and np.abs(pages[0][2]).sum() > 0          # values are copies
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads, dk, dv", [(3, 24, 40), (2, 128, 128), (1, 200, 16), (2, 64, 256), (1, 33, 4)])
+def test_gla_step_of_one_token_a_sequence(ops, dtype, heads, dk, dv):
+    """The fused step against the plain recurrence, norm and gate, from states that are not zero, on slots in
+    another order than the sequences; and against the scan kernel with the separate norm and gate."""
+    assert ops.gla_step_fits(dk, dv)
+    rng = np.random.default_rng(dk + dv)
+    B, tau = 3, 2.5
+    proj = t(rng.normal(size=(B, 3 + 2 * heads * dk + 2 * heads * dv)), dtype)          # 3 unused | q | k | v | g
+    q_off, k_off, v_off = 3, 3 + heads * dk, 3 + 2 * heads * dk
+    g_off = v_off + heads * dv
+    z, zb = rng.normal(size=(B, heads * dk)) * 3, rng.normal(size=heads * dk)
+    slots = [5, 0, 3]
+    state0 = rng.normal(size=(6, heads, dk, dv))
+    gain = rng.normal(size=dv)
+    state = t(state0)
+    got = ops.gla_step(proj, q_off, k_off, v_off, g_off, t(z), t(zb), tau, dk ** -0.5, state, t(slots, torch.int32), t(gain),
+                       1e-5, heads, dk, dv)
+    p = f64(proj)
+    alpha = Z.sigmoid(f64(t(z)) + f64(t(zb))) ** (1.0 / tau)
+    want_state = state0.astype(np.float32).astype(np.float64)
+    o = np.zeros((B, heads, dv))
+    for b in range(B):
+        for h in range(heads):
+            o[b, h] = Z.gla_recurrence(p[b:b + 1, q_off + h * dk:q_off + (h + 1) * dk] * dk ** -0.5,
+                                       p[b:b + 1, k_off + h * dk:k_off + (h + 1) * dk],
+                                       p[b:b + 1, v_off + h * dv:v_off + (h + 1) * dv],
+                                       alpha[b:b + 1, h * dk:(h + 1) * dk], want_state[slots[b], h])[0]
+    want = Z.rms_norm(o, gain, 1e-5) * Z.silu(p[:, g_off:g_off + heads * dv].reshape(B, heads, dv))
+    close(state, want_state, 5e-6, "state")
+    close(got, want.reshape(B, -1), 1e-5 if dtype == torch.float32 else BF16_OUT, "step")
+    assert ops.gla_step_fits(512, 512) is False and ops.gla_step_fits(64, 30) is False
 
 
 def test_gla_token_by_token_is_the_scan(ops):
