@@ -19,7 +19,7 @@
 #define GLA_SLICES 16
 #define GLA_MAX_ROWS 32          // rows of a column per thread: dim <= 16 * 32
 #define GLA_MAX_NB 32            // tokens of a block
-#define GLA_STAGE 16             // staged elements of q, k and z per thread and block: nb * dim <= 16 * 256
+#define GLA_STAGE 16             // most staged elements of q, k and z per thread and block: nb * dim <= 16 * 256 (STAGE: 4 or 16)
 #define GLA_VSTAGE (GLA_MAX_NB * GLA_COLS / 256)
 
 __device__ __forceinline__ float log_sigmoid(float z) {
@@ -35,7 +35,7 @@ __global__ void gla_decay_kernel(float* __restrict__ z, const float* __restrict_
     z[e] = expf(log_sigmoid(z[e] + (z_bias ? z_bias[e % width] : 0.f)) * inv_tau);
 }
 
-template <typename TA, bool V4>
+template <typename TA, int RPT, int STAGE>
 __global__ void __launch_bounds__(256)
 gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, int q_off, int k_off, int v_off,
                 const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau, float q_scale,
@@ -59,34 +59,47 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
 
     // a block's inputs on their way: every load is issued whatever the indices are, from a token and a column
     // pulled back inside the data
-    float rq[GLA_STAGE], rk[GLA_STAGE], rz[GLA_STAGE], rv[GLA_VSTAGE];
+    float rq[STAGE], rk[STAGE], rz[STAGE], rv[GLA_VSTAGE];
+    // which token of a block and which channel each staged element is: the same for every block, worked out once
+    // (a division a token would cost more than the token's arithmetic)
+    int s_tok[STAGE], s_ch[STAGE], v_tok[GLA_VSTAGE], v_col[GLA_VSTAGE];
+#pragma unroll
+    for (int j = 0; j < STAGE; ++j) {
+        const int e = min(tid + j * 256, per - 1);
+        s_tok[j] = e / dim;
+        s_ch[j] = e - s_tok[j] * dim;
+    }
+#pragma unroll
+    for (int j = 0; j < GLA_VSTAGE; ++j) {
+        const int e = min(tid + j * 256, nb * GLA_COLS - 1);
+        v_tok[j] = e / GLA_COLS;
+        v_col[j] = min(col0 + e % GLA_COLS, vdim - 1);
+    }
     auto ask = [&](int tb) {
 #pragma unroll
-        for (int j = 0; j < GLA_STAGE; ++j) {
+        for (int j = 0; j < STAGE; ++j) {
             if (j * 256 >= per) break;                       // (per is the same for all: no thread has an element here)
-            const int e = min(tid + j * 256, per - 1);
-            const int tok = min(tb + e / dim, t1 - 1), i = e % dim;
-            const TA* x = proj + (size_t)tok * row;
-            rq[j] = to_f32(x[q_off + h * dim + i]);
-            rk[j] = to_f32(x[k_off + h * dim + i]);
+            const int tok = min(tb + s_tok[j], t1 - 1), i = s_ch[j];
+            const TA* x = proj + (size_t)tok * row + h * dim + i;
+            rq[j] = to_f32(x[q_off]);
+            rk[j] = to_f32(x[k_off]);
             rz[j] = z[((size_t)tok * heads + h) * dim + i];
         }
 #pragma unroll
         for (int j = 0; j < GLA_VSTAGE; ++j) {
-            const int e = min(tid + j * 256, nb * GLA_COLS - 1);
-            const int tok = min(tb + e / GLA_COLS, t1 - 1), cc = min(col0 + e % GLA_COLS, vdim - 1);
-            rv[j] = to_f32(proj[(size_t)tok * row + v_off + h * vdim + cc]);
+            if (j * 256 >= nb * GLA_COLS) break;
+            const int tok = min(tb + v_tok[j], t1 - 1);
+            rv[j] = to_f32(proj[(size_t)tok * row + v_off + h * vdim + v_col[j]]);
         }
     };
     auto put = [&](int which) {
         float* buf = lds + (size_t)which * nb * stride;
 #pragma unroll
-        for (int j = 0; j < GLA_STAGE; ++j) {
-            const int e = tid + j * 256;
+        for (int j = 0; j < STAGE; ++j) {
             if (j * 256 >= per) break;
-            if (e < per) {
-                const int i = e % dim;
-                float* at = buf + (size_t)(e / dim) * stride;
+            if (tid + j * 256 < per) {
+                const int i = s_ch[j];
+                float* at = buf + (size_t)s_tok[j] * stride;
                 at[i] = rq[j] * q_scale;
                 at[dim + i] = rk[j];
                 at[2 * dim + i] = z_is_decay ? rz[j] : expf(log_sigmoid(rz[j] + (z_bias ? z_bias[h * dim + i] : 0.f)) * inv_tau);
@@ -95,7 +108,7 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
 #pragma unroll
         for (int j = 0; j < GLA_VSTAGE; ++j) {
             const int e = tid + j * 256;
-            if (e < nb * GLA_COLS) buf[(size_t)(e / GLA_COLS) * stride + 3 * dim + e % GLA_COLS] = rv[j];
+            if (e < nb * GLA_COLS) buf[(size_t)v_tok[j] * stride + 3 * dim + e % GLA_COLS] = rv[j];
         }
     };
     ask(t0);
@@ -106,15 +119,16 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
         const bool more = tb + nb < t1;                      // the same for the whole workgroup
         if (more) ask(tb + nb);
         const float* buf = lds + (size_t)(blk & 1) * nb * stride;
-        for (int n = 0; n < nb; ++n) {
-            if (tb + n >= t1) break;                         // the same for the whole workgroup
-            const float* at = buf + (size_t)n * stride;
+        // eight tokens at a time: their state updates follow one another, but nothing else of a token waits for
+        // the token before, so the LDS reads run ahead and the slices' shares meet (two shuffles a token) after the
+        // eight, side by side (a workgroup's four wavefronts are one a SIMD: nothing else hides a latency here)
+        auto token = [&](const float* at) -> float {
             const float v = at[3 * dim + c];
             float o = 0.f;
-            if (V4) {                                        // rpt a multiple of 4 and every slice whole: 16 bytes a read
+            if (RPT > 0) {                                   // dim = 16 RPT, RPT a multiple of 4: 16 bytes a read, no guards
 #pragma unroll
-                for (int j = 0; j < GLA_MAX_ROWS; j += 4) {
-                    if (j < rpt) {
+                for (int j = 0; j < (RPT > 0 ? RPT : 4); j += 4) {
+                    {
                         const float4 q4 = *reinterpret_cast<const float4*>(at + row0 + j);
                         const float4 k4 = *reinterpret_cast<const float4*>(at + dim + row0 + j);
                         const float4 a4 = *reinterpret_cast<const float4*>(at + 2 * dim + row0 + j);
@@ -135,10 +149,31 @@ gla_scan_kernel(float* __restrict__ out, const TA* __restrict__ proj, int row, i
                     }
                 }
             }
-            // lanes of a wavefront: 4 slices x 16 columns
-            o += __shfl_xor(o, 16, RI_WAVE);
-            o += __shfl_xor(o, 32, RI_WAVE);
-            if ((tid & (RI_WAVE - 1)) < GLA_COLS) part[blk & 1][n][wave][c] = o;
+            return o;
+        };
+        for (int n0 = 0; n0 < nb; n0 += 8) {
+            if (tb + n0 >= t1) break;                        // the same for the whole workgroup
+            float oo[8];
+            if (n0 + 8 <= nb && tb + n0 + 8 <= t1) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) oo[u] = token(buf + (size_t)(n0 + u) * stride);
+            } else {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    oo[u] = 0.f;
+                    if (n0 + u < nb && tb + n0 + u < t1) oo[u] = token(buf + (size_t)(n0 + u) * stride);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {                    // lanes of a wavefront: 4 slices x 16 columns
+                oo[u] += __shfl_xor(oo[u], 16, RI_WAVE);
+                oo[u] += __shfl_xor(oo[u], 32, RI_WAVE);
+            }
+            if ((tid & (RI_WAVE - 1)) < GLA_COLS) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (n0 + u < nb) part[blk & 1][n0 + u][wave][c] = oo[u];
+            }
         }
         if (more) put((blk + 1) & 1);
         __syncthreads();
@@ -168,11 +203,14 @@ extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row,
     RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "gla_scan: dtype %d", act_dtype);
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((vdim + GLA_COLS - 1) / GLA_COLS, heads, seqs);
-    // tokens a block: as many as the staging registers hold (dim <= 512: at least eight), at most 32; 16 where
-    // the workgroups outnumber the compute units, so that several fit one unit's LDS; a step of single tokens 1
+    // tokens a block: as many as the staging registers hold (dim <= 512: at least eight), at most 32; 16 and 8
+    // where the workgroups outnumber the compute units, so that several fit one unit's LDS and hide one another's
+    // waits; a step of single tokens 1
     int nb = GLA_STAGE * 256 / dim;
     nb = nb > GLA_MAX_NB ? GLA_MAX_NB : nb;
-    if (nb > 16 && (long)grid.x * grid.y * grid.z > ri_compute_units()) nb = 16;
+    const long wgs = (long)grid.x * grid.y * grid.z, cus = ri_compute_units();
+    if (nb > 16 && wgs > cus) nb = 16;
+    if (nb > 8 && wgs > 3 * cus) nb = 8;
     if (tokens == seqs) nb = 1;
     const size_t lds = (size_t)2 * nb * (3 * dim + GLA_COLS) * sizeof(float);
     // a prompt: the decays of all its tokens in one pass, in place of z, before the walk
@@ -183,22 +221,36 @@ extern "C" int ri_gla_scan(float* out, const void* proj, int act_dtype, int row,
         gla_decay_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(z, z_bias, 1.0f / tau, total, heads * dim);
         z_is_decay = 1;
     }
-    const bool v4 = dim % (4 * GLA_SLICES) == 0;             // every slice has a multiple of 4 rows, 16-byte aligned in LDS
+    // key heads of 64, 128, 256 or 512: a thread's rows are a fixed number, a multiple of 4, read 16 bytes at a time
+    const int fixed = (dim == 64 || dim == 128 || dim == 256 || dim == 512) ? dim / GLA_SLICES : 0;
     // (more than 64 KB of dynamic LDS has to be asked for, once for every form of the kernel)
-#define RI_GLA_GO(T, V)                                                                                              \
+#define RI_GLA_GO(T, V, G)                                                                                           \
     if (lds > 48 * 1024) {                                                                                           \
         static bool asked = false;                                                                                   \
         if (!asked) {                                                                                                \
-            hipError_t e_ = hipFuncSetAttribute((const void*)gla_scan_kernel<T, V>,                                  \
+            hipError_t e_ = hipFuncSetAttribute((const void*)gla_scan_kernel<T, V, G>,                               \
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);             \
             RI_REQUIRE(e_ == hipSuccess, "gla_scan: %s", hipGetErrorString(e_));                                     \
             asked = true;                                                                                            \
         }                                                                                                            \
     }                                                                                                                \
-    gla_scan_kernel<T, V><<<grid, 256, lds, s>>>(out, (const T*)proj, row, q_off, k_off, v_off, z, z_bias, 1.0f / tau,   \
+    gla_scan_kernel<T, V, G><<<grid, 256, lds, s>>>(out, (const T*)proj, row, q_off, k_off, v_off, z, z_bias, 1.0f / tau,   \
                                                  q_scale, state, cu_seqlens, slots, heads, dim, vdim, nb, z_is_decay)
-    if (act_dtype == RI_F32) { if (v4) { RI_GLA_GO(float, true); } else { RI_GLA_GO(float, false); } }
-    else                     { if (v4) { RI_GLA_GO(bf16_t, true); } else { RI_GLA_GO(bf16_t, false); } }
+    // (blocks of up to 4 * 256 staged elements run with a quarter of the staging registers: more wavefronts a SIMD)
+    const bool few = (long)nb * dim <= 4 * 256;
+#define RI_GLA_STAGE(T, R)                                                                                           \
+    if (few) { RI_GLA_GO(T, R, 4); } else { RI_GLA_GO(T, R, 16); }
+#define RI_GLA_ROWS(T)                                                                                               \
+    switch (fixed) {                                                                                                 \
+        case 4: RI_GLA_STAGE(T, 4) break;                                                                            \
+        case 8: RI_GLA_STAGE(T, 8) break;                                                                            \
+        case 16: RI_GLA_STAGE(T, 16) break;                                                                          \
+        case 32: RI_GLA_STAGE(T, 32) break;                                                                          \
+        default: RI_GLA_STAGE(T, 0) break;                                                                           \
+    }
+    if (act_dtype == RI_F32) { RI_GLA_ROWS(float) } else { RI_GLA_ROWS(bf16_t) }
+#undef RI_GLA_ROWS
+#undef RI_GLA_STAGE
 #undef RI_GLA_GO
     RI_LAUNCH_CHECK("gla_scan");
     return 0;

@@ -257,7 +257,9 @@ def test_the_matrix_core_kernels_cap_their_scores(ops, form, dh, heads, kv_heads
 # ---------------------------------------------------------------- gated linear attention
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads, dk, dv, lens", [(3, 24, 40, [19, 1, 8]), (2, 72, 16, [5]), (1, 200, 17, [3, 2]),
-                                                  (2, 64, 32, [9, 2]), (1, 128, 16, [20, 1])])
+                                                  (2, 64, 32, [9, 2]), (1, 128, 16, [20, 1]),
+                                                  # enough (sequence, head, column tile) triples for 8 and for 16 columns a workgroup
+                                                  (8, 16, 32, [2, 1] * 16), (8, 16, 32, [1, 3] * 32)])
 def test_gla_scan_and_output_gate(ops, dtype, heads, dk, dv, lens):
     rng = np.random.default_rng(dk)
     T = sum(lens)
@@ -268,8 +270,8 @@ def test_gla_scan_and_output_gate(ops, dtype, heads, dk, dv, lens):
     g_off = v_off + heads * dv
     z = rng.normal(size=(T, heads * dk)) * 3
     zb = rng.normal(size=heads * dk)
-    slots = [4, 0, 2][:len(lens)]
-    state0 = rng.normal(size=(6, heads, dk, dv))
+    slots = [4, 0, 2][:len(lens)] if len(lens) <= 3 else list(rng.permutation(len(lens) + 3)[:len(lens)])
+    state0 = rng.normal(size=(max(6, len(lens) + 3), heads, dk, dv))
     state = t(state0)
     cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     o = ops.gla_scan(proj, q_off, k_off, v_off, t(z), t(zb), tau, dk ** -0.5, state, t(cu, torch.int32),
