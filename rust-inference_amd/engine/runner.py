@@ -21,7 +21,7 @@ from ..sampling import DEFAULT_SEED
 
 
 def build_parser() -> argparse.ArgumentParser:
-    ap = argparse.ArgumentParser(prog="runner", description="Text generation with a Qwen3 checkpoint on one MI355X")
+    ap = argparse.ArgumentParser(prog="runner", description="Text generation with a model folder (any registered architecture) on one MI355X")
     ap.add_argument("model_dir", help="HuggingFace checkpoint directory (config.json, *.safetensors, tokenizer.json)")
     ap.add_argument("-p", "--prompt", action="append", help="prompt text or token ids; read from stdin when omitted")
     ap.add_argument("--prompt-ids", action="append", help="a prompt as comma-separated token ids")
