@@ -14,7 +14,7 @@
 #include "api.h"
 #include "common.h"
 
-#define ST_MAX_STREAMS 8
+#define ST_MAX_STREAMS 16
 
 enum { ST_NORM_NONE = 0, ST_NORM_RMS = 1, ST_NORM_LAYER = 2 };
 

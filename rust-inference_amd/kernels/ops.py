@@ -327,7 +327,7 @@ def qk_norm_temper_kv_write(qkv, q_gain, k_gain, eps: float, temper, tok_pos, to
 
 
 NORM_NONE, NORM_RMS, NORM_LAYER = 0, 1, 2
-MAX_STREAMS = 8
+MAX_STREAMS = 16
 
 
 def streams_read_norm(streams, pending, mix, out_coef, in_coef, gain, bias, eps: float, norm_kind: int, out_dtype,

@@ -62,7 +62,7 @@ BF16_OUT = 7.5e-3
 
 
 # ---------------------------------------------------------------- streams and norms
-@pytest.mark.parametrize("streams, dim", [(4, 104), (1, 200), (3, 72), (8, 40)])
+@pytest.mark.parametrize("streams, dim", [(4, 104), (1, 200), (3, 72), (8, 40), (2, 70), (16, 33), (4, 5000)])
 @pytest.mark.parametrize("kind", ["layer", "rms", "none"])
 def test_streams_write_read_and_norm(ops, streams, dim, kind):
     rng = np.random.default_rng(streams * 100 + dim)
