@@ -248,3 +248,46 @@ def test_a_sequence_cannot_outgrow_the_positions_the_model_has(folders):
         engine.step([StepEntry(slot, [1] * (Z_C["max_positions"] + 1), "last")])
     cache.release(slot)
     cache.check_consistent()
+
+
+def drawn_config(seed):
+    """A configuration drawn at random: sizes, head counts, order and number of layers, the looped stretch, the
+    constants, with and without streams, cap, temperature and feed-forward."""
+    rng = np.random.default_rng(1000 + seed)
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+    layers = []
+    for _ in range(int(rng.integers(2, 6))):
+        ff = pick([None, 40, 72, 136])
+        if rng.random() < 0.6:
+            kv = pick([1, 2, 3, 4])
+            dim = pick([8, 16, 24, 32, 48, 64, 128])
+            layers.append(attention(kv * pick([1, 2, 4]), kv, dim, pick([dim, dim, 8, 40, 64]), float(rng.uniform(0.05, 0.4)),
+                                    pick([None, 3.0, 15.0, 50.0]),
+                                    pick([None, {"coef": float(rng.uniform(0.05, 1.0)), "every": pick([1, 3, 32, 64])}]), ff))
+        else:
+            layers.append(gla(pick([1, 2, 5]), pick([8, 24, 32, 64, 128]), pick([4, 16, 24, 64, 128]), float(rng.uniform(1.0, 20.0)),
+                              pick([3, 8, 12, 16]), ff))
+    cfg = {"architecture": "Zidepel", "vocab": int(rng.integers(50, 400)), "width": pick([48, 80, 136, 192]),
+           "max_positions": 320, "norm": {"eps": pick([1e-5, 1e-6, 1e-3])}, "layers": layers}
+    if rng.random() < 0.75:
+        cfg["streams"] = pick([1, 2, 3, 4, 6])
+    if rng.random() < 0.7:
+        a = int(rng.integers(0, len(layers)))
+        cfg["loop"] = {"start": a, "stop": int(rng.integers(a, len(layers) + 1)), "times": pick([1, 2, 3])}
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    from rust_inference_amd.parts import load_model
+    from rust_inference_amd.weights import write_random_model
+    cfg = drawn_config(seed)
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed, torch.bfloat16, matrix_std=0.12, gain_std=0.1)
+    rng = np.random.default_rng(seed)
+    reqs = {f"r{i}": [int(t) for t in rng.integers(0, cfg["vocab"], n)] for i, n in enumerate((150, 37, 1, 66))}
+    batch = {rid: (toks, max(1, len(toks) - 9)) for rid, toks in reqs.items()}
+    for dtype_name in ("float32", "bfloat16"):
+        model = load_model(folder, DTYPES[dtype_name])
+        for what, steps in (("whole", plans.whole(reqs)), ("last 32 one by one", plans.tail_one_by_one(reqs, 32)),
+                            ("a batch", plans.unequal_batches([batch])), ("portions", in_portions(reqs, [33, 2, 64]))):
+            against_plain(folder, replay(model, steps), reqs, dtype_name, f"configuration {seed}, {what}")
