@@ -217,7 +217,8 @@ class GroupedQueryAttention(Mixer):
                                         self.head_dim, self.v_dim, ctx.cu_seqlens, ctx.max_new)
         with profiler.section(profiler.ATTENTION):
             o = self.attend(qkv, ctx, store, page_table)
-        return self.project_out(o, link)
+        with profiler.section(profiler.OUT_PROJECTION):          # float32 into the residual: one rounding less a layer
+            return self.rt.linear_packed(o, self.w_o, out_dtype=torch.float32, parts_ok=True, link=link)
 
     def project_out(self, o, link):
         with profiler.section(profiler.OUT_PROJECTION):

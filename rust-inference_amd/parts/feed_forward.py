@@ -85,4 +85,5 @@ class ReluSquaredFF(FeedForward):
         rt = self.rt
         with profiler.section(profiler.MLP):
             a = ops.relu_squared(ops.as_rows(rt.linear_packed(x, self.w_up)))
-            return rt.linear_packed(a, self.w_down, parts_ok=True)      # may come in parts: the stream's next read adds them
+            # float32 into the residual (or in parts that the stream's next read adds): the sum is never rounded to 16 bits
+            return rt.linear_packed(a, self.w_down, out_dtype=torch.float32, parts_ok=True)

@@ -80,10 +80,10 @@ class GatedLinearAttention(Mixer):
                 y = ops.gla_step(proj, 0, hk, 2 * hk, 2 * hk + hv, z, self.z_bias, self.tau, self.dim ** -0.5, store,
                                  ctx.slots, self.gain, self.eps, self.heads, self.dim, self.vdim)
             with profiler.section(profiler.OUT_PROJECTION):
-                return rt.linear_packed(y, self.w_o, parts_ok=True)
+                return rt.linear_packed(y, self.w_o, out_dtype=torch.float32, parts_ok=True)
         with profiler.section(profiler.ATTENTION):
             o = ops.gla_scan(proj, 0, hk, 2 * hk, z, self.z_bias, self.tau, self.dim ** -0.5, store, ctx.cu_seqlens,
                              ctx.slots, self.heads, self.dim, self.vdim)
             y = ops.gla_norm_gate(o, proj, 2 * hk + hv, self.gain, self.eps, self.heads, self.vdim)
         with profiler.section(profiler.OUT_PROJECTION):
-            return rt.linear_packed(y, self.w_o, parts_ok=True)
+            return rt.linear_packed(y, self.w_o, out_dtype=torch.float32, parts_ok=True)
