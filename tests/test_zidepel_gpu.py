@@ -300,3 +300,21 @@ def test_configurations_drawn_at_random(tmp_path, seed):
             for rid, toks in reqs.items():
                 err = rel_to_max(got[rid], plain_logits(folder, toks))
                 assert err <= 8e-2, f"configuration {seed}, {what}, request {rid}: error {err:.3e} of the largest logit (bfloat16)"
+
+
+def test_the_command_line_generates_what_the_plain_implementation_does(folders):
+    """bin/runner on a Zidepel folder, prompts as token ids: greedy in float32, sections timed, and a seeded
+    temperature run that gives the same tokens twice."""
+    cfg, w = read_model_f64(folders["A"])
+    prompts = list(requests_for("A", [9, 14], 8).values())
+    want = [Z.greedy(cfg, w, p, 6)[0] for p in prompts]
+    base = [sys.executable, os.path.join(ROOT, "bin", "runner"), folders["A"], "--dtype", "float32", "-n", "6"]
+    two = subprocess.run(base + ["--prompt-ids", ",".join(map(str, prompts[0])), "--prompt-ids", ",".join(map(str, prompts[1])),
+                                 "--profile"], capture_output=True, text=True, timeout=300)
+    assert two.returncode == 0, two.stderr[-2000:]
+    assert [[int(t) for t in ln.split()] for ln in two.stdout.strip().splitlines()] == want
+    assert "section " in two.stderr and "attention" in two.stderr
+    drawn = [subprocess.run(base + ["-p", " ".join(map(str, prompts[0])), "--temperature", "0.9", "--top-k", "20", "--seed", "5"],
+                            capture_output=True, text=True, timeout=300) for _ in range(2)]
+    assert drawn[0].returncode == 0, drawn[0].stderr[-2000:]
+    assert drawn[0].stdout == drawn[1].stdout and len(drawn[0].stdout.split()) == 6

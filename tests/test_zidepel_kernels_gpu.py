@@ -254,6 +254,35 @@ def test_the_matrix_core_kernels_cap_their_scores(ops, form, dh, heads, kv_heads
     close(same, want, BF16_OUT, "the generic kernel on the same pages")
 
 
+@pytest.mark.parametrize("cap", [None, 2.5])
+def test_the_matrix_core_kernels_find_one_far_key(ops, cap):
+    """1,500 keys in bfloat16, the one that matters 1,400 back, behind five chunk borders: the last token alone (the
+    one-token kernels) and the whole prompt (the prompt kernel).  Uncapped the output is that key's value row."""
+    rng = np.random.default_rng(11)
+    n, dh = 1500, 64
+    m = {"heads": 2, "kv_heads": 1, "dim": dh, "vdim": dh, "scale": 1.0, "softcap": cap, "q_temp": None}
+    k, v, q = rng.normal(size=(n, 1, dh)) * 0.1, rng.normal(size=(n, 1, dh)), rng.normal(size=(n, 2, dh)) * 0.1
+    k[97, 0] = 0.0
+    k[97, 0, 9] = 6.0
+    q[-1] = 0.0
+    q[-1, :, 9] = 6.0
+    qkv, kp, vp, tok_pos, tok_seq, table = paged(ops, m, q, k, v, [n], torch.bfloat16)
+    r = f64(qkv)
+    ops.qk_norm_temper_kv_write(qkv, None, None, 1e-5, None, tok_pos, tok_seq, table, kp, vp, 2, 1, dh, dh)
+    want = Z.attention_core(m, r[:, :2 * dh].reshape(n, 2, dh), r[:, 2 * dh:3 * dh].reshape(n, 1, dh),
+                            r[:, 3 * dh:].reshape(n, 1, dh), np.arange(n)).reshape(n, -1)
+    whole = ops.attention_prefill_bf16(qkv, kp, vp, t([0, n], torch.int32), tok_pos, table, 1, n, 2, 1, dh, None, 1.0, cap)
+    last = ops.attention_decode_bf16(guarded(qkv[-1:].clone()), kp, vp, t([0, 1], torch.int32), t([n - 1], torch.int32), table,
+                                     1, n, 2, 1, dh, None, 1.0, softcap=cap)
+    close(whole, want, BF16_OUT, "prompt")
+    close(last, want[-1:], BF16_OUT, "one token")
+    far = f64(t(v[97, 0], torch.bfloat16))
+    if cap is None:
+        assert np.abs(f64(last)[0, :dh] - far).max() < 2e-2
+    else:
+        assert np.abs(f64(last)[0, :dh] - far).max() > 0.1
+
+
 # ---------------------------------------------------------------- gated linear attention
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads, dk, dv, lens", [(3, 24, 40, [19, 1, 8]), (2, 72, 16, [5]), (1, 200, 17, [3, 2]),
