@@ -336,6 +336,76 @@ embed_positions_norm_kernel(float* __restrict__ out, const TT* __restrict__ tabl
     }
 }
 
+// The same with a row's 8- or 16-byte pieces asked for up front (rows of up to 8192 elements, a multiple of 4): a
+// step of one token is then two trips to memory (the id and position, the rows), not one per element.
+template <typename TT, int VPT>
+__global__ void __launch_bounds__(256)
+embed_positions_norm_vec_kernel(float* __restrict__ out, const TT* __restrict__ table, const TT* __restrict__ positions,
+                                const int32_t* __restrict__ ids, const int32_t* __restrict__ tok_pos,
+                                const float* __restrict__ gain, const float* __restrict__ bias, float eps, int kind,
+                                int dim) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x;
+    const TT* a = table + (size_t)ids[t] * dim;
+    const TT* b = positions ? positions + (size_t)tok_pos[t] * dim : a;      // (no positions: the load is made and dropped)
+    float4 u[VPT];
+    int col[VPT];
+    bool ok[VPT];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = (threadIdx.x + i * 256) * 4;
+        ok[i] = c < dim;
+        col[i] = ok[i] ? c : 0;
+    }
+    float4 ra[VPT], rb[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        ra[i] = ld4(a + col[i]);
+        rb[i] = ld4(b + col[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        float4 r = positions ? make_float4(ra[i].x + rb[i].x, ra[i].y + rb[i].y, ra[i].z + rb[i].z, ra[i].w + rb[i].w) : ra[i];
+        if (!ok[i]) r = make_float4(0.f, 0.f, 0.f, 0.f);
+        u[i] = r;
+        sum += kind == ST_NORM_RMS ? (r.x * r.x + r.y * r.y) + (r.z * r.z + r.w * r.w) : (r.x + r.y) + (r.z + r.w);
+    }
+    float mean = 0.f, inv = 1.f;
+    if (kind != ST_NORM_NONE) {
+        const float total = block_sum(sum, scratch);
+        if (kind == ST_NORM_RMS) {
+            inv = 1.0f / sqrtf(total / (float)dim + eps);
+        } else {
+            mean = total / (float)dim;
+            float dev = 0.f;
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                if (ok[i]) {
+                    const float x0 = u[i].x - mean, x1 = u[i].y - mean, x2 = u[i].z - mean, x3 = u[i].w - mean;
+                    dev += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
+                }
+            }
+            inv = 1.0f / sqrtf(block_sum(dev, scratch) / (float)dim + eps);
+        }
+    }
+    float* o = out + (size_t)t * dim;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        if (!ok[i]) continue;
+        float4 v = u[i];
+        if (kind != ST_NORM_NONE) {
+            const float4 g = ld4(gain + col[i]);
+            v = make_float4((v.x - mean) * inv * g.x, (v.y - mean) * inv * g.y, (v.z - mean) * inv * g.z, (v.w - mean) * inv * g.w);
+            if (bias) {
+                const float4 bb = ld4(bias + col[i]);
+                v = make_float4(v.x + bb.x, v.y + bb.y, v.z + bb.z, v.w + bb.w);
+            }
+        }
+        st4(o + col[i], v);
+    }
+}
+
 extern "C" int ri_embed_positions_norm(float* out, const void* table, const void* positions, int table_dtype,
                                        const int32_t* ids, const int32_t* tok_pos, const float* gain,
                                        const float* bias, float eps, int norm_kind, int tokens, int dim, void* stream) {
@@ -345,6 +415,19 @@ extern "C" int ri_embed_positions_norm(float* out, const void* table, const void
     RI_REQUIRE(norm_kind == ST_NORM_NONE || gain != nullptr, "embed_positions_norm: a norm needs its gain");
     RI_REQUIRE(table_dtype == RI_F32 || table_dtype == RI_BF16, "embed_positions_norm: table dtype %d", table_dtype);
     hipStream_t s = (hipStream_t)stream;
+    if (dim % 4 == 0 && dim <= 8192) {
+#define RI_EMBED_VEC(T, VPT)                                                                                          \
+    embed_positions_norm_vec_kernel<T, VPT><<<tokens, 256, 0, s>>>(out, (const T*)table, (const T*)positions, ids, tok_pos,  \
+                                                                   gain, bias, eps, norm_kind, dim)
+#define RI_EMBED_DIM(T)                                                                                               \
+    if (dim <= 1024) RI_EMBED_VEC(T, 1); else if (dim <= 2048) RI_EMBED_VEC(T, 2); else if (dim <= 4096) RI_EMBED_VEC(T, 4); \
+    else RI_EMBED_VEC(T, 8)
+        if (table_dtype == RI_F32) { RI_EMBED_DIM(float); } else { RI_EMBED_DIM(bf16_t); }
+#undef RI_EMBED_DIM
+#undef RI_EMBED_VEC
+        RI_LAUNCH_CHECK("embed_positions_norm");
+        return 0;
+    }
     const size_t lds = (size_t)dim * sizeof(float);
     if (table_dtype == RI_F32)
         embed_positions_norm_kernel<float><<<tokens, 256, lds, s>>>(out, (const float*)table, (const float*)positions, ids,

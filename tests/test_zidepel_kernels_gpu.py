@@ -119,10 +119,11 @@ def test_streams_start_from_one_row_and_the_plain_residual_is_one_stream(ops):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_embedding_with_positions_and_norm(ops, dtype):
+@pytest.mark.parametrize("dim", [136, 70, 2052])
+def test_embedding_with_positions_and_norm(ops, dtype, dim):
     rng = np.random.default_rng(1)
-    table, pos = t(rng.normal(size=(300, 136)), dtype), t(rng.normal(size=(50, 136)), dtype)
-    gain, bias = rng.normal(size=136), rng.normal(size=136)
+    table, pos = t(rng.normal(size=(300, dim)), dtype), t(rng.normal(size=(50, dim)), dtype)
+    gain, bias = rng.normal(size=dim), rng.normal(size=dim)
     ids, where = [299, 0, 7, 7], [0, 49, 3, 4]
     cfg = {"norm": {"eps": 1e-5}}
     w = {"embed": f64(table), "pos": f64(pos), "embed.norm": gain, "embed.norm.b": bias}
