@@ -51,11 +51,12 @@ int ri_qk_norm_rope_kv_write(void* qkv, int act_dtype, const float* q_gain, cons
 // per sequence).  q is read from qkv rows (row stride q_stride elements); out: [tokens, heads * head_dim].
 // window <= 0: all keys 0..pos; else keys max(0, pos - window + 1)..pos.  v_dim: the size of a value head
 // (v_pages: [pages, kv_heads, v_dim, page_size]; out: [tokens, heads * v_dim]).  softcap > 0: a score s becomes
-// softcap * tanh(s / softcap) before the softmax.
+// softcap * tanh(s / softcap) before the softmax.  slopes (float32 [heads] or NULL): a distance bias, the score of
+// query head h at position p for the key at position j becomes s - slopes[h] * (p - j).
 int ri_attention(void* out, const void* q, int act_dtype, int q_stride, const void* k_pages, const void* v_pages,
                  int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table,
                  int table_width, int tokens, int heads, int kv_heads, int head_dim, int v_dim, int page_size,
-                 int window, float scale, float softcap, void* stream);
+                 int window, float scale, float softcap, const float* slopes, void* stream);
 
 // Queries and keys for an attention without rotation, keys and values into their pages, from the fused
 // projection qkv: [tokens, heads * dim + kv_heads * dim + kv_heads * vdim].  Per-head RMS norm of q and k (gains
@@ -111,8 +112,40 @@ int ri_gla_step(void* out, const void* proj, int act_dtype, int row, int q_off, 
                 const float* z, const float* z_bias, float tau, float q_scale, float* state, const int32_t* slots,
                 const float* gain, float eps, int seqs, int heads, int dim, int vdim, void* stream);
 
+// The gated delta rule.  proj: [tokens, row] of act_dtype with the projections of q and k (kv_heads heads of dim each)
+// and v (heads heads of vdim) side by side from column q_off on: `channels` = 2 kv_heads dim + heads vdim columns.
+// ri_delta_prepare: per channel the causal convolution over time with taps [channels, ntaps] (last column: the
+// current token's) and silu, the inputs before a step's first token taken from tails [slots, ntaps - 1, channels]
+// (float32; zeros at a sequence's start); q and k made unit vectors per head (x / sqrt(sum x^2 + 1e-6)), q also
+// times dim^(-1/2); qkv: float32 [tokens, channels].  gates: float32 [tokens, 2 heads]: g = exp(-exp(a_log) *
+// softplus(a + dt_bias)) then beta = sigmoid(b), from ab [tokens, 2 heads] (a then b).  Then the tails are moved on
+// by the step's tokens.
+int ri_delta_prepare(float* qkv, float* gates, const void* proj, int act_dtype, int row, int q_off, const float* taps,
+                     int ntaps, float* tails, const float* ab, const float* a_log, const float* dt_bias,
+                     const int32_t* tok_seq, const int32_t* cu_seqlens, const int32_t* slots, int seqs, int tokens,
+                     int heads, int kv_heads, int dim, int vdim, void* stream);
+// Per sequence and head, over the sequence's new tokens in order: S <- g S; u = beta (v - S^T k); S <- S + k u^T;
+// o = S^T q.  state: float32 [slots, heads, dim, vdim]; out: float32 [tokens, heads * vdim].
+int ri_delta_max_dim();
+int ri_delta_scan(float* out, const float* qkv, const float* gates, float* state, const int32_t* cu_seqlens,
+                  const int32_t* slots, int seqs, int tokens, int heads, int kv_heads, int dim, int vdim, void* stream);
+
+// A mixture of experts' router.  z: float32 [tokens, experts] router logits; s = sigmoid(z); the `top` experts with
+// the largest s + correction (the lower index on a tie) are chosen; their weights are their s divided by the sum of
+// the chosen s (+ 1e-20).  ids: int32 [tokens, top] in the order chosen; weights: float32 [tokens, top]; dense:
+// float32 [tokens, experts], the weight of every expert, zero where it was not chosen.
+int ri_experts_route(int32_t* ids, float* weights, float* dense, const float* z, const float* correction, int tokens,
+                     int experts, int top, void* stream);
+// The experts' activation on the gate and up branches of all experts side by side: gu [tokens, experts, 2, ff]
+// (gate then up); g = min(gate, limit), u = clamp(up, -limit, limit);
+// out[t, e, i] = dense[t, e] * g * sigmoid(1.702 g) * (u + 1), zero for experts that the token did not choose.
+int ri_experts_activate(void* out, const void* gu, int dtype, const float* dense, int tokens, int experts, int ff,
+                        float limit, void* stream);
+
 // out[i] = max(y[i], 0)^2.
 int ri_relu_squared(void* out, const void* y, int dtype, long total, void* stream);
+// out[i] = 0.5 y (1 + tanh(sqrt(2 / pi) (y + 0.044715 y^3))), in float32.
+int ri_gelu_tanh(void* out, const void* y, int dtype, long total, void* stream);
 
 // The same attention on the matrix cores, for bfloat16, pages of 32 tokens and head_dim 32, 64 or 128.
 // Prefill form: any number of new tokens per sequence (cu_seqlens: int32 [seqs + 1] over the flat tokens,

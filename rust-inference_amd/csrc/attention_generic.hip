@@ -3,7 +3,8 @@
 // One workgroup per (token, query head); keys in tiles of 256 that start at multiples of 256, so the
 // order of every sum depends on the key's position alone, never on how tokens were cut into steps.
 //
-// score_j = (q . k_j) * scale, then, with a cap c > 0, score_j <- c tanh(score_j / c); the query at position p
+// score_j = (q . k_j) * scale, then, with a cap c > 0, score_j <- c tanh(score_j / c), then, with a slope per
+// query head, score_j <- score_j - slope_h (p - j); the query at position p
 // sees keys lo..p with lo = 0 or p - window + 1;
 // online softmax with running maximum m, running sum l and factor exp(m_old - m_new)
 // (the reference: src/attention.rs:117-149; its GPU form src/cuda/kernels.cu:345-405).
@@ -47,7 +48,7 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
                          const TC* __restrict__ v_pages, const int32_t* __restrict__ tok_pos,
                          const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ page_table, int table_width,
                          int heads, int kv_heads, int head_dim, int v_dim, int page_size, int window, float scale,
-                         float softcap) {
+                         float softcap, const float* __restrict__ slopes) {
     extern __shared__ float qs[];                 // head_dim floats: the query
     __shared__ float ps[ATT_TILE];                // this tile's weights
     __shared__ long rowoff[ATT_TILE];             // element offset of each key's column in the value pool
@@ -57,6 +58,7 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
     const int kvh = h / (heads / kv_heads);       // consecutive query heads share a kv head
     const int qpos = tok_pos[t];
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
+    const float slope = slopes ? slopes[h] : 0.f;
     const int32_t* table = page_table + (size_t)tok_seq[t] * table_width;
 
     for (int d = tid; d < head_dim; d += ATT_TILE) qs[d] = to_f32(q[(size_t)t * q_stride + (size_t)h * head_dim + d]);
@@ -85,6 +87,7 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
             }
             s = dot * scale;
             if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+            if (slopes) s -= slope * (float)(qpos - j);
         }
         const float m_new = fmaxf(m, block_max(s, scratch));
         const float p = valid ? expf(s - m_new) : 0.f;
@@ -114,17 +117,17 @@ template <typename T, bool VEC>
 static void launch_attention(void* out, const void* q, int q_stride, const void* k_pages, const void* v_pages,
                              const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table,
                              int table_width, int tokens, int heads, int kv_heads, int head_dim, int v_dim,
-                             int page_size, int window, float scale, float softcap, hipStream_t s) {
+                             int page_size, int window, float scale, float softcap, const float* slopes, hipStream_t s) {
     attention_generic_kernel<T, T, VEC><<<dim3(tokens, heads), ATT_TILE, (size_t)head_dim * sizeof(float), s>>>(
         (T*)out, (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, tok_pos, tok_seq, page_table,
-        table_width, heads, kv_heads, head_dim, v_dim, page_size, window, scale, softcap);
+        table_width, heads, kv_heads, head_dim, v_dim, page_size, window, scale, softcap, slopes);
 }
 
 extern "C" int ri_attention(void* out, const void* q, int act_dtype, int q_stride, const void* k_pages,
                             const void* v_pages, int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq,
                             const int32_t* page_table, int table_width, int tokens, int heads, int kv_heads,
                             int head_dim, int v_dim, int page_size, int window, float scale, float softcap,
-                            void* stream) {
+                            const float* slopes, void* stream) {
     RI_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                "attention: tokens %d, heads %d, kv heads %d", tokens, heads, kv_heads);
     RI_REQUIRE(head_dim >= 1 && head_dim <= ATT_MAX_HEAD_DIM, "attention: head_dim %d must be between 1 and %d", head_dim,
@@ -142,7 +145,7 @@ extern "C" int ri_attention(void* out, const void* q, int act_dtype, int q_strid
     const bool vec = head_dim % (act_dtype == RI_F32 ? 4 : 8) == 0 && (uintptr_t)k_pages % 16 == 0;
 #define RI_ATT_GO(T, V) launch_attention<T, V>(out, q, q_stride, k_pages, v_pages, tok_pos, tok_seq, page_table, \
                                                table_width, tokens, heads, kv_heads, head_dim, v_dim, page_size, window, scale, \
-                                               softcap, s)
+                                               softcap, slopes, s)
     if (act_dtype == RI_F32) { if (vec) RI_ATT_GO(float, true); else RI_ATT_GO(float, false); }
     else                     { if (vec) RI_ATT_GO(bf16_t, true); else RI_ATT_GO(bf16_t, false); }
 #undef RI_ATT_GO

@@ -313,44 +313,63 @@ extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int in
     return 0;
 }
 
-// ------------------------------------------------------------------ squared ReLU
-// out[i] = max(y[i], 0)^2, the square taken in float32.
-template <typename T>
-__global__ void relu_squared_kernel(T* __restrict__ out, const T* __restrict__ y, long total) {
-    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= total) return;
-    const float v = fmaxf(to_f32(y[e]), 0.f);
-    from_f32(out + e, v * v);
+// ------------------------------------------------------------------ activations of a dense feed-forward
+// out[i] = act(y[i]), taken in float32.  ACT_RELU2: max(y, 0)^2.  ACT_GELU_TANH: the tanh form of GELU,
+// 0.5 y (1 + tanh(sqrt(2 / pi) (y + 0.044715 y^3))).
+enum { ACT_RELU2 = 0, ACT_GELU_TANH = 1 };
+
+template <int ACT>
+__device__ __forceinline__ float activate(float v) {
+    if (ACT == ACT_RELU2) {
+        const float r = fmaxf(v, 0.f);
+        return r * r;
+    }
+    return 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
 }
 
-__global__ void relu_squared_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ y, long total8) {
+template <typename T, int ACT>
+__global__ void activation_kernel(T* __restrict__ out, const T* __restrict__ y, long total) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    from_f32(out + e, activate<ACT>(to_f32(y[e])));
+}
+
+template <int ACT>
+__global__ void activation_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ y, long total8) {
     const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= total8) return;
     const uint4 g = *reinterpret_cast<const uint4*>(y + e * 8);
     const uint32_t gw[4] = {g.x, g.y, g.z, g.w};
     uint32_t o[4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        const float a = fmaxf(__uint_as_float(gw[k] << 16), 0.f), b = fmaxf(__uint_as_float(gw[k] & 0xFFFF0000u), 0.f);
-        o[k] = pack_bf16x2(a * a, b * b);
-    }
+    for (int k = 0; k < 4; ++k)
+        o[k] = pack_bf16x2(activate<ACT>(__uint_as_float(gw[k] << 16)), activate<ACT>(__uint_as_float(gw[k] & 0xFFFF0000u)));
     *reinterpret_cast<uint4*>(out + e * 8) = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
-extern "C" int ri_relu_squared(void* out, const void* y, int dtype, long total, void* stream) {
-    RI_REQUIRE(total > 0, "relu_squared: %ld elements", total);
-    RI_REQUIRE((total + 255) / 256 <= 2147483647L, "relu_squared: %ld elements exceed one launch", total);
+template <int ACT>
+static int launch_activation(const char* name, void* out, const void* y, int dtype, long total, void* stream) {
+    RI_REQUIRE(total > 0, "%s: %ld elements", name, total);
+    RI_REQUIRE((total + 255) / 256 <= 2147483647L, "%s: %ld elements exceed one launch", name, total);
     hipStream_t s = (hipStream_t)stream;
     if (dtype == RI_F32)
-        relu_squared_kernel<float><<<(unsigned)((total + 255) / 256), 256, 0, s>>>((float*)out, (const float*)y, total);
+        activation_kernel<float, ACT><<<(unsigned)((total + 255) / 256), 256, 0, s>>>((float*)out, (const float*)y, total);
     else if (dtype == RI_BF16 && total % 8 == 0 && (uintptr_t)y % 16 == 0 && (uintptr_t)out % 16 == 0)
-        relu_squared_bf16x8_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, total / 8);
+        activation_bf16x8_kernel<ACT><<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, total / 8);
     else if (dtype == RI_BF16)
-        relu_squared_kernel<bf16_t><<<(unsigned)((total + 255) / 256), 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, total);
+        activation_kernel<bf16_t, ACT><<<(unsigned)((total + 255) / 256), 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, total);
     else
-        RI_REQUIRE(false, "relu_squared: dtype %d", dtype);
-    RI_LAUNCH_CHECK("relu_squared");
+        RI_REQUIRE(false, "%s: dtype %d", name, dtype);
+    RI_LAUNCH_CHECK(name);
     return 0;
+}
+
+extern "C" int ri_relu_squared(void* out, const void* y, int dtype, long total, void* stream) {
+    return launch_activation<ACT_RELU2>("relu_squared", out, y, dtype, total, stream);
+}
+
+extern "C" int ri_gelu_tanh(void* out, const void* y, int dtype, long total, void* stream) {
+    return launch_activation<ACT_GELU_TANH>("gelu_tanh", out, y, dtype, total, stream);
 }
 
 // ------------------------------------------------------------------ bias

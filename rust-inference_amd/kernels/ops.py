@@ -27,7 +27,7 @@ _SIGNATURES = {
                                  c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                  c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
-                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
+                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_void_p],
     "ri_qk_norm_temper_kv_write": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_float, c_int, c_void_p, c_void_p,
                                    c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                    c_int, c_int, c_int, c_int, c_void_p],
@@ -43,6 +43,14 @@ _SIGNATURES = {
     "ri_gla_norm_gate": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_int, c_int, c_int,
                          c_void_p],
     "ri_relu_squared": [c_void_p, c_void_p, c_int, ctypes.c_long, c_void_p],
+    "ri_gelu_tanh": [c_void_p, c_void_p, c_int, ctypes.c_long, c_void_p],
+    "ri_delta_prepare": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_delta_max_dim": [],
+    "ri_delta_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                      c_void_p],
+    "ri_experts_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ri_experts_activate": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
     "ri_attention_prefill_bf16": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
     "ri_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -287,10 +295,11 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, 
 
 
 def attention(qkv, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, kv_heads: int, head_dim: int,
-              window: int | None, scale: float, softcap: float | None = None) -> torch.Tensor:
+              window: int | None, scale: float, softcap: float | None = None, slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of every new token over its sequence's pages; q is the first ``H dh`` columns of ``qkv``.
     The size of a value head is read from ``v_pages [pages, kv_heads, v_dim, page]``; with ``softcap`` a score
-    ``s`` becomes ``softcap * tanh(s / softcap)`` before the softmax."""
+    ``s`` becomes ``softcap * tanh(s / softcap)`` before the softmax; with ``slopes`` (float32 ``[heads]``) the score of
+    head ``h`` at position ``p`` for the key at ``j`` then loses ``slopes[h] * (p - j)``."""
     tokens, stride = qkv.shape
     v_dim = v_pages.shape[2]
     if tuple(k_pages.shape[:2]) != tuple(v_pages.shape[:2]) or k_pages.shape[2] != v_pages.shape[3] or k_pages.shape[3] != head_dim:
@@ -300,7 +309,7 @@ def attention(qkv, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, k
           _dev(v_pages, "v_pages"), code(k_pages.dtype), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
           _dev(tok_seq, "tok_seq", torch.int32, (tokens,)), _dev(page_table, "page_table", torch.int32),
           page_table.shape[1], tokens, heads, kv_heads, head_dim, v_dim, k_pages.shape[2], int(window or 0),
-          float(scale), float(softcap or 0.0), _stream())
+          float(scale), float(softcap or 0.0), _opt(slopes, "slopes", torch.float32, (heads,)), _stream())
     return out
 
 
@@ -432,6 +441,91 @@ def relu_squared(y: torch.Tensor) -> torch.Tensor:
     out = torch.empty(y.shape, dtype=y.dtype, device=y.device)
     if y.numel():
         _call("ri_relu_squared", _dev(out, "out"), _dev(y, "y"), code(y.dtype), y.numel(), _stream())
+    return out
+
+
+def gelu_tanh(y: torch.Tensor) -> torch.Tensor:
+    """``0.5 y (1 + tanh(sqrt(2 / pi) (y + 0.044715 y^3)))`` elementwise, taken in float32."""
+    out = torch.empty(y.shape, dtype=y.dtype, device=y.device)
+    if y.numel():
+        _call("ri_gelu_tanh", _dev(out, "out"), _dev(y, "y"), code(y.dtype), y.numel(), _stream())
+    return out
+
+
+ACTIVATIONS = {"relu2": relu_squared, "gelu_tanh": gelu_tanh}      # what a dense feed-forward may name
+
+DELTA_MAX_DIM = 256
+DELTA_MAX_TAPS = 16
+
+
+def delta_prepare(proj, q_off: int, taps, tails, ab, a_log, dt_bias, tok_seq, cu_seqlens, slots, heads: int,
+                  kv_heads: int, dim: int, vdim: int):
+    """What the gated delta rule's walk reads, for all tokens of a step: float32 ``qkv [T, channels]`` (q and k of
+    ``kv_heads`` heads of ``dim``, v of ``heads`` heads of ``vdim``: the projections at column ``q_off`` of ``proj``
+    through their short convolutions (``taps [channels, K]``, the inputs before the step from ``tails [slots, K - 1,
+    channels]``) and silu, q and k as unit vectors per head, q times ``dim^(-1/2)``) and ``gates [T, 2 heads]``
+    (``g = exp(-exp(a_log) softplus(a + dt_bias))`` then ``beta = sigmoid(b)`` from ``ab [T, 2 heads]``).  The tails
+    are moved on by the step's tokens."""
+    tokens, row = proj.shape
+    seqs = slots.shape[0]
+    channels = 2 * kv_heads * dim + heads * vdim
+    ntaps = taps.shape[1]
+    if tails.dim() != 3 or tuple(tails.shape[1:]) != (ntaps - 1, channels):
+        raise ShapeError(f"the convolutions' tails are {list(tails.shape)}, not [slots, {ntaps - 1}, {channels}]")
+    qkv = torch.empty((tokens, channels), dtype=torch.float32, device=proj.device)
+    gates = torch.empty((tokens, 2 * heads), dtype=torch.float32, device=proj.device)
+    _call("ri_delta_prepare", _dev(qkv, "qkv"), _dev(gates, "gates"), _dev(proj, "proj"), code(proj.dtype), row, q_off,
+          _dev(taps, "taps", torch.float32, (channels, ntaps)), ntaps, _dev(tails, "tails", torch.float32),
+          _dev(ab, "ab", torch.float32, (tokens, 2 * heads)), _dev(a_log, "a_log", torch.float32, (heads,)),
+          _dev(dt_bias, "dt_bias", torch.float32, (heads,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
+          seqs, tokens, heads, kv_heads, dim, vdim, _stream())
+    return qkv, gates
+
+
+def delta_scan(qkv, gates, state, cu_seqlens, slots, heads: int, kv_heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """The gated delta rule over every sequence's new tokens, ``S <- g S; u = beta (v - S^T k); S <- S + k u^T;
+    o = S^T q``; float32 ``[T, heads * vdim]``.  ``state: [slots, heads, dim, vdim]`` float32 is read and written at
+    the sequences' slots."""
+    tokens = qkv.shape[0]
+    seqs = slots.shape[0]
+    channels = 2 * kv_heads * dim + heads * vdim
+    if state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, vdim):
+        raise ShapeError(f"the state is {list(state.shape)}, not [slots, {heads}, {dim}, {vdim}]")
+    out = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=qkv.device)
+    _call("ri_delta_scan", _dev(out, "out"), _dev(qkv, "qkv", torch.float32, (tokens, channels)),
+          _dev(gates, "gates", torch.float32, (tokens, 2 * heads)), _dev(state, "state", torch.float32),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
+          seqs, tokens, heads, kv_heads, dim, vdim, _stream())
+    return out
+
+
+EXPERTS_MAX = 1024
+
+
+def experts_route(z: torch.Tensor, correction: torch.Tensor, top: int):
+    """The router of a mixture of experts from its float32 logits ``z [T, E]``: ``s = sigmoid(z)``, the ``top``
+    experts with the largest ``s + correction`` (the lower index on a tie), weights ``s / (sum of the chosen s +
+    1e-20)``.  Returns ``ids [T, top]`` int32, ``weights [T, top]`` and ``dense [T, E]`` (zero where not chosen)."""
+    tokens, experts = z.shape
+    ids = torch.empty((tokens, top), dtype=torch.int32, device=z.device)
+    weights = torch.empty((tokens, top), dtype=torch.float32, device=z.device)
+    dense = torch.empty((tokens, experts), dtype=torch.float32, device=z.device)
+    _call("ri_experts_route", _dev(ids, "ids"), _dev(weights, "weights"), _dev(dense, "dense"),
+          _dev(z, "z", torch.float32), _dev(correction, "correction", torch.float32, (experts,)), tokens, experts,
+          int(top), _stream())
+    return ids, weights, dense
+
+
+def experts_activate(gu: torch.Tensor, dense: torch.Tensor, ff: int, limit: float) -> torch.Tensor:
+    """``dense[t, e] * g sigmoid(1.702 g) (u + 1)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``
+    for ``gu [T, E * 2 * ff]`` (every expert's gate then up); ``[T, E * ff]``, zero for experts not chosen."""
+    tokens, experts = dense.shape
+    if tuple(gu.shape) != (tokens, experts * 2 * ff):
+        raise ShapeError(f"gate|up rows are {list(gu.shape)} for {experts} experts of {ff}")
+    out = torch.empty((tokens, experts * ff), dtype=gu.dtype, device=gu.device)
+    _call("ri_experts_activate", _dev(out, "out"), _dev(gu, "gu"), code(gu.dtype), _dev(dense, "dense", torch.float32),
+          tokens, experts, ff, float(limit), _stream())
     return out
 
 

@@ -43,7 +43,9 @@ class GroupedQueryAttention(Mixer):
     head where it is not ``head_dim`` (the output product then reads ``heads * v_dim``); ``scale`` replaces
     ``1 / sqrt(head_dim)``; ``softcap = c`` turns a score ``s`` into ``c tanh(s / c)`` before the softmax;
     ``q_temper = (coef, every)`` multiplies the normed query at position ``p`` by
-    ``1 + coef * ln(floor((p + 1) / every) + 1)``, all in float32.  ``names`` gives the checkpoint names of
+    ``1 + coef * ln(floor((p + 1) / every) + 1)``, all in float32; ``distance_slopes`` (one per query head) takes
+    ``slope_h * (i - j)`` off the score of the query at position ``i`` for the key at ``j``, after scale and cap;
+    ``window`` holds on this path as on the other.  ``names`` gives the checkpoint names of
     ``q, k, v, o, q_norm, k_norm`` where they are not ``<prefix>q_proj.weight`` and so on.  A mixer with any of
     ``v_dim``, ``softcap`` or ``q_temper`` takes no position encoding; its q/k norm, temperature and cache write
     are one kernel (``ops.qk_norm_temper_kv_write``).
@@ -54,7 +56,8 @@ class GroupedQueryAttention(Mixer):
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, prefix: str, qk_norm: bool = True,
                  eps: float = 1e-6, position: PartSpec | None = None, window: int | None = None,
                  qkv_bias: bool = False, o_bias: bool = False, v_dim: int | None = None, scale: float | None = None,
-                 softcap: float | None = None, q_temper: tuple | None = None, names: dict | None = None):
+                 softcap: float | None = None, q_temper: tuple | None = None, names: dict | None = None,
+                 distance_slopes: tuple | None = None):
         if heads < 1 or kv_heads < 1 or heads % kv_heads:
             raise ConfigError(f"{heads} attention heads not divisible by {kv_heads} kv heads")
         if not 1 <= head_dim <= ops.MAX_HEAD_DIM:
@@ -73,7 +76,11 @@ class GroupedQueryAttention(Mixer):
         if self.q_temper is not None and self.q_temper[1] < 1:
             raise ConfigError(f"a query temperature every {self.q_temper[1]} positions")
         # what the rotary kernels do not know goes through the kernels that do
-        self.tempered = self.v_dim != head_dim or self.q_temper is not None
+        # a distance bias: the score of head h at position i for the key at j loses distance_slopes[h] * (i - j)
+        self.distance_slopes = tuple(float(v) for v in distance_slopes) if distance_slopes is not None else None
+        if self.distance_slopes is not None and len(self.distance_slopes) != heads:
+            raise ConfigError(f"{len(self.distance_slopes)} distance slopes for {heads} heads")
+        self.tempered = self.v_dim != head_dim or self.q_temper is not None or self.distance_slopes is not None
         self.position = build_part("position", position or PartSpec("none"))
         if (self.tempered or self.softcap is not None) and (position is not None and position.kind != "none"):
             raise ConfigError("an attention with a score cap, a query temperature or value heads of their own size "
@@ -120,6 +127,8 @@ class GroupedQueryAttention(Mixer):
         if self.o_bias:
             self.b_o = rt.place_gain(weights[p + "o_proj.bias"])
         self.position.bind(weights, rt)
+        self.slopes = (torch.tensor(self.distance_slopes, dtype=torch.float32, device=rt.device)
+                       if self.distance_slopes is not None else None)
 
     def bind_plain(self, weights):
         if self.tempered or self.softcap is not None:
@@ -232,8 +241,10 @@ class GroupedQueryAttention(Mixer):
         args = (self.heads, self.kv_heads, self.head_dim, self.window, self.scale)
         group = self.heads // self.kv_heads
         cap = self.softcap
-        if self.v_dim != self.head_dim:          # value heads of their own size: the generic kernel alone takes them
-            return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args, cap)
+        slopes = getattr(self, "slopes", None)
+        if self.v_dim != self.head_dim or slopes is not None:
+            # value heads of their own size, a distance bias: the generic kernel alone takes them
+            return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args, cap, slopes)
         if self.rt.invariant:
             # one kernel for prompts and single tokens alike: in the prompt kernel a token's sums run over its
             # sequence's pages in order whatever the other rows of its tile are (a page that a row does not

@@ -4,6 +4,7 @@ from __future__ import annotations
 import torch
 
 from .. import profiler
+from ..errors import ConfigError
 from ..kernels import ops
 from ..weights.loader import MATRIX, TensorSpec
 from .base import FeedForward
@@ -60,13 +61,16 @@ class SwiGLU(FeedForward):
             return rt.linear_packed(a, self.w_down, parts_ok=True, link=link)
 
 
-@register_part("feed_forward", "relu2")
-class ReluSquaredFF(FeedForward):
-    """``down(relu(up(x))^2)``, no gate and no bias; ``names`` gives the checkpoint names of ``up`` and ``down``
-    where they are not ``<prefix>up_proj.weight`` and ``<prefix>down_proj.weight``."""
+@register_part("feed_forward", "dense")
+class DenseFF(FeedForward):
+    """``down(act(up(x)))``, no gate and no bias; ``activation`` is one of ``ops.ACTIVATIONS`` (``"relu2"``:
+    ``max(z, 0)^2``; ``"gelu_tanh"``: the tanh form of GELU).  ``names`` gives the checkpoint names of ``up`` and
+    ``down`` where they are not ``<prefix>up_proj.weight`` and ``<prefix>down_proj.weight``."""
 
-    def __init__(self, hidden: int, inter: int, prefix: str, names: dict | None = None):
-        self.hidden, self.inter, self.prefix = hidden, inter, prefix
+    def __init__(self, hidden: int, inter: int, prefix: str, names: dict | None = None, activation: str = "relu2"):
+        if activation not in ops.ACTIVATIONS:
+            raise ConfigError(f"activation {activation!r} is not one of {', '.join(sorted(ops.ACTIVATIONS))}")
+        self.hidden, self.inter, self.prefix, self.activation = hidden, inter, prefix, activation
         self.names = {"up": prefix + "up_proj.weight", "down": prefix + "down_proj.weight"}
         self.names.update(names or {})
 
@@ -84,6 +88,14 @@ class ReluSquaredFF(FeedForward):
     def forward(self, x, ctx):
         rt = self.rt
         with profiler.section(profiler.MLP):
-            a = ops.relu_squared(ops.as_rows(rt.linear_packed(x, self.w_up)))
+            a = ops.ACTIVATIONS[self.activation](ops.as_rows(rt.linear_packed(x, self.w_up)))
             # float32 into the residual (or in parts that the stream's next read adds): the sum is never rounded to 16 bits
             return rt.linear_packed(a, self.w_down, out_dtype=torch.float32, parts_ok=True)
+
+
+@register_part("feed_forward", "relu2")
+class ReluSquaredFF(DenseFF):
+    """``down(relu(up(x))^2)``: the dense feed-forward with the squared ReLU."""
+
+    def __init__(self, hidden: int, inter: int, prefix: str, names: dict | None = None):
+        super().__init__(hidden, inter, prefix, names, "relu2")

@@ -26,12 +26,14 @@ register_part("stream", "residual", ResidualStream)
 
 @register_part("connection", "hyper")
 class HyperConnection(Part):
-    """The coefficients of one sublayer: tensors ``<prefix>in``, ``<prefix>mix`` and ``<prefix>out``."""
+    """The coefficients of one sublayer: tensors ``<prefix>in``, ``<prefix>mix`` and ``<prefix>out``.
+    ``out_scale``: a constant of the model on every sublayer's output, ``x_t <- sum_s mix[s, t] x_s + out_scale *
+    out[t] * y``; it is multiplied into ``out`` (in float32) when the weights are bound."""
 
-    def __init__(self, streams: int, prefix: str):
+    def __init__(self, streams: int, prefix: str, out_scale: float = 1.0):
         if not 1 <= streams <= ops.MAX_STREAMS:
             raise ConfigError(f"{streams} residual streams: the kernel takes 1 to {ops.MAX_STREAMS}")
-        self.streams, self.prefix = streams, prefix
+        self.streams, self.prefix, self.out_scale = streams, prefix, float(out_scale)
 
     def tensors(self):
         n, p = self.streams, self.prefix
@@ -41,6 +43,22 @@ class HyperConnection(Part):
         self.rt = rt
         p = self.prefix
         self.read, self.write, self.mix = (rt.place_gain(weights[p + k]) for k in ("in", "out", "mix"))
+        if self.out_scale != 1.0:
+            self.write = (self.write * torch.tensor(self.out_scale, dtype=torch.float32, device=self.write.device)).contiguous()
+
+
+@register_part("connection", "scaled_add")
+class ScaledAdd(Part):
+    """The connection of a sublayer to one plain residual, ``x <- x + scale * y``, in the terms of the streams'
+    kernel: one stream that is read and kept as it is.  It has no tensors."""
+
+    def __init__(self, scale: float = 1.0):
+        self.streams, self.scale = 1, float(scale)
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.read = self.mix = None                                   # taken as 1 by the kernel
+        self.write = torch.tensor([self.scale], dtype=torch.float32, device=rt.device)
 
 
 @register_part("stream", "hyper")
