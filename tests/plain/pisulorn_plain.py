@@ -161,12 +161,18 @@ def dense_ff(mlp, w, pre, h):
     return gelu_tanh(h @ w[pre + "up"].T) @ w[pre + "down"].T
 
 
+ROUTE_MARGINS = None      # a list: route() then notes, per call, every token's gap between the last expert chosen and the best one left out
+
+
 def route(mlp, w, pre, h):
     """Chosen experts ``[T, top]`` and their weights ``[T, top]``: sigmoid scores, the choice by score plus
     correction, the weights from the scores alone, normalised."""
     s = sigmoid(h @ w[pre + "router"].T)
     choice = s + w[pre + "correction"]
     top = mlp["router"]["top"]
+    if ROUTE_MARGINS is not None and top < choice.shape[-1]:
+        ranked = -np.sort(-choice, axis=-1)
+        ROUTE_MARGINS.append(ranked[:, top - 1] - ranked[:, top])
     chosen = np.argsort(-choice, axis=-1, kind="stable")[:, :top]
     picked = np.take_along_axis(s, chosen, -1)
     return chosen, picked / (picked.sum(-1, keepdims=True) + 1e-20)
