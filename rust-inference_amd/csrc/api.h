@@ -147,13 +147,14 @@ int ri_relu_squared(void* out, const void* y, int dtype, long total, void* strea
 // out[i] = 0.5 y (1 + tanh(sqrt(2 / pi) (y + 0.044715 y^3))), in float32.
 int ri_gelu_tanh(void* out, const void* y, int dtype, long total, void* stream);
 
-// The same attention on the matrix cores, for bfloat16, pages of 32 tokens and head_dim 32, 64 or 128.
+// The same attention on the matrix cores, for bfloat16, pages of 32 tokens and head_dim 32, 64 or 128 (softcap and
+// slopes as in ri_attention; slopes NULL: no distance bias).
 // Prefill form: any number of new tokens per sequence (cu_seqlens: int32 [seqs + 1] over the flat tokens,
 // max_new: the most new tokens of any sequence); at most 64 query heads per kv head.
 int ri_attention_prefill_bf16(void* out, const void* qkv, int q_stride, const void* k_pages, const void* v_pages,
                               const int32_t* cu_seqlens, const int32_t* tok_pos, const int32_t* page_table,
                               int table_width, int seqs, int max_new, int heads, int kv_heads, int head_dim,
-                              int page_size, int window, float scale, float softcap, void* stream);
+                              int page_size, int window, float scale, float softcap, const float* slopes, void* stream);
 // (softcap > 0, here and in the decode form: a score s becomes softcap * tanh(s / softcap) before the softmax)
 
 // Decode form: exactly one new token per sequence; keys in chunks of 256 (in a step of few workgroups each cut into
@@ -171,7 +172,7 @@ int ri_attention_decode_bf16(void* out, float* workspace, const void* qkv, int q
                              const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
                              const int32_t* page_table, int table_width, int seqs, int max_chunks, int heads,
                              int kv_heads, int head_dim, int page_size, int window, float scale, float softcap,
-                             int tiled_out, void* stream);
+                             const float* slopes, int tiled_out, void* stream);
 
 // tiled_out (both decode forms): the result [seqs, heads * head_dim] is written in the matrix cores' operand order
 // (see tiled_at in common.h) for the packed product that reads it.

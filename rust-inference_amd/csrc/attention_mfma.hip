@@ -119,6 +119,10 @@ struct Columns {
     // follows still multiplies by the scale: (q . k) <- cap_post * tanh((q . k) * cap_pre), cap_pre = scale / c,
     // cap_post = c / scale; both 0: no cap
     float cap_pre, cap_post;
+    // a distance bias: the score of a column at position p for the key at j loses slope (p - j); bias is the
+    // column's slope over the scale, so that it too acts on the raw products; all 0 (biased false): none
+    float bias[NT];
+    bool biased;
 };
 
 // tanh through one exponential: 1 - 2 / (e^(2x) + 1), exact at both ends (e^(2x) = inf or 0).
@@ -130,6 +134,12 @@ __device__ __forceinline__ float tanh_by_exp(float x) {
 __device__ __forceinline__ void cap_scores(float (&s)[8], float cap_pre, float cap_post) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) s[e] = cap_post * tanh_by_exp(s[e] * cap_pre);
+}
+
+// key0: the position of the first of the lane's eight keys.
+__device__ __forceinline__ void bias_scores(float (&s)[8], float bias, int qpos, int key0) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s[e] -= bias * (float)(qpos - key0 - e);
 }
 
 // One page for NT tiles of columns, in two halves so that the key fragments and the value fragments
@@ -153,6 +163,7 @@ __device__ __forceinline__ void scores_and_weights(Columns<DH, NT>& c, const Fra
         }
         float s[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
         if (c.cap_pre != 0.f) cap_scores(s, c.cap_pre, c.cap_post);
+        if (c.biased) bias_scores(s, c.bias[j], c.qpos[j], key0);
         if (!open) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -219,6 +230,8 @@ __device__ __forceinline__ void init_columns(Columns<DH, NT>& c) {
         c.qpos[j] = -1;
         c.lo[j] = 0;
         c.cap_pre = c.cap_post = 0.f;
+        c.bias[j] = 0.f;
+        c.biased = false;
 #pragma unroll
         for (int ks = 0; ks < DH / 32; ++ks) c.q[j][ks].u = make_uint4(0, 0, 0, 0);
 #pragma unroll
@@ -229,7 +242,8 @@ __device__ __forceinline__ void init_columns(Columns<DH, NT>& c) {
 // The same work in four pieces, for a loop that takes the scores of the next page while it weighs this one
 // (the prefill's): the results are those of scores_and_weights and weighted_values bit for bit.
 template <int DH, int NT>
-__device__ __forceinline__ void scores_of(const Columns<DH, NT>& c, const Frag (&kf)[2][DH / 32], float (&s)[NT][8]) {
+__device__ __forceinline__ void scores_of(const Columns<DH, NT>& c, const Frag (&kf)[2][DH / 32], float (&s)[NT][8],
+                                          int page, int lane) {
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
         floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -244,6 +258,7 @@ __device__ __forceinline__ void scores_of(const Columns<DH, NT>& c, const Frag (
             s[j][4 + e] = s1[e];
         }
         if (c.cap_pre != 0.f) cap_scores(s[j], c.cap_pre, c.cap_post);
+        if (c.biased) bias_scores(s[j], c.bias[j], c.qpos[j], page * PAGE + (lane >> 4) * 8);
     }
 }
 
@@ -363,7 +378,8 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                          const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ tok_pos,
                          const int32_t* __restrict__ page_table, int table_width, int heads, int kv_heads,
-                         int window, float scale_log2, float cap_pre, float cap_post) {
+                         int window, float scale_log2, float cap_pre, float cap_post,
+                         const float* __restrict__ slopes, float inv_scale) {
     __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][PAGE * LdsPage<DH>::KS];
     __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][DH * LdsPage<DH>::VS];
     const int lane = threadIdx.x & 63;
@@ -384,11 +400,13 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
     init_columns<DH, NT>(c);
     c.cap_pre = cap_pre;
     c.cap_post = cap_post;
+    c.biased = slopes != nullptr;
     const int jg = lane >> 4;
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
         const int col = j * 16 + (lane & 15);
         const int tl = col / group, g = col - tl * group;
+        if (slopes) c.bias[j] = slopes[kvh * group + g] * inv_scale;
         if (tl < nt) {
             const int tok = t0 + tl;
             c.qpos[j] = tok_pos[tok];
@@ -453,7 +471,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
         RI_TURN_LOADS(p_lo - 1);
         Frag kf[2][DH / 32];
         key_frags_from_lds<DH>(kf, k_lds[0], lane);
-        scores_of<DH, NT>(c, kf, s_cur);
+        scores_of<DH, NT>(c, kf, s_cur, p_lo, lane);
         if (!RI_PAGE_OPEN(p_lo)) mask_scores<DH, NT>(c, s_cur, p_lo, lane);
         maxima_with<DH, NT>(c, s_cur, m_new, scale_log2);
         move_reference<DH, NT>(c, m_new, ref);
@@ -469,7 +487,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
         {
             Frag kf[2][DH / 32];
             key_frags_from_lds<DH>(kf, k_lds[i & 1], lane);
-            scores_of<DH, NT>(c, kf, s_next);
+            scores_of<DH, NT>(c, kf, s_next, p + 1, lane);
             weights_of<DH, NT>(c, s_cur, ref, w, scale_log2);
         }
         if (decltype(masked)::value) mask_scores<DH, NT>(c, s_next, p + 1, lane);
@@ -528,7 +546,8 @@ __global__ void __launch_bounds__(CW * 64)
 attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, int q_stride,
                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
-                        int heads, int kv_heads, int window, float scale_log2, int max_chunks, float cap_pre, float cap_post) {
+                        int heads, int kv_heads, int window, float scale_log2, int max_chunks, float cap_pre, float cap_post,
+                        const float* __restrict__ slopes, float inv_scale) {
     __shared__ float o_lds[CW][DH * 17];           // [d * 17 + col]: no bank conflicts either way
     __shared__ float ml_lds[CW][2][16];
     const int lane = threadIdx.x & 63;
@@ -553,6 +572,10 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
     c.cap_pre = cap_pre;
     c.cap_post = cap_post;
     const int jg = lane >> 4, col = lane & 15;
+    if (slopes) {
+        c.biased = true;
+        c.bias[0] = slopes[kvh * group + min(col, group - 1)] * inv_scale;
+    }
     {
         const bf16_t* qp = qkv + (long)tok * q_stride + (kvh * group + min(col, group - 1)) * DH + jg * 8;
 #pragma unroll
@@ -835,7 +858,8 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
                           const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
                           const float* __restrict__ inv_freq, bf16_t* k_pages, bf16_t* v_pages,
                           const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
-                          int heads, int kv_heads, int window, float scale_log2, int splits, int tiled, float cap_pre, float cap_post) {
+                          int heads, int kv_heads, int window, float scale_log2, int splits, int tiled, float cap_pre, float cap_post,
+                          const float* __restrict__ slopes, float inv_scale) {
     static_assert(!FUSED || DH <= 128, "one (d, d + DH/2) pair per lane");
     __shared__ float o_lds[W][DH * 17];
     __shared__ float ml_lds[W][2][16];
@@ -889,6 +913,10 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
     c.cap_pre = cap_pre;
     c.cap_post = cap_post;
     const int jg = lane >> 4, col = lane & 15;
+    if (slopes) {
+        c.biased = true;
+        c.bias[0] = slopes[kvh * (heads / kv_heads) + min(col, heads / kv_heads - 1)] * inv_scale;
+    }
     fetch_table(0);
     if (FUSED) {
         const bf16_t* row = qkv + (long)b * q_stride;
@@ -1217,7 +1245,7 @@ extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_strid
                                          const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
                                          const int32_t* page_table, int table_width, int seqs, int max_new,
                                          int heads, int kv_heads, int head_dim, int page_size, int window,
-                                         float scale, float softcap, void* stream) {
+                                         float scale, float softcap, const float* slopes, void* stream) {
     const float cap_pre = softcap > 0.f ? scale / softcap : 0.f, cap_post = softcap > 0.f ? softcap / scale : 0.f;
     RI_REQUIRE(scale > 0.f, "attention_prefill_bf16: the scale %g must be positive", (double)scale);
     if (check_common("attention_prefill_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width)) return 1;
@@ -1237,7 +1265,7 @@ extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_strid
         attn_prefill_mfma_kernel<DH, NT><<<grid, 256, 0, s>>>(                                                   \
             (bf16_t*)out, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,          \
             cu_seqlens, tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, cap_pre,          \
-            cap_post);                                                                                           \
+            cap_post, slopes, 1.f / scale);                                                                      \
         break;
     switch (head_dim * 8 + nt_tiles) {
         RI_PREFILL_CASE(32, 4)
@@ -1282,7 +1310,8 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
                                         const void* k_pages, const void* v_pages, const int32_t* cu_seqlens,
                                         const int32_t* tok_pos, const int32_t* page_table, int table_width, int seqs,
                                         int max_chunks, int heads, int kv_heads, int head_dim, int page_size,
-                                        int window, float scale, float softcap, int tiled_out, void* stream) {
+                                        int window, float scale, float softcap, const float* slopes, int tiled_out,
+                                        void* stream) {
     const float cap_pre = softcap > 0.f ? scale / softcap : 0.f, cap_post = softcap > 0.f ? softcap / scale : 0.f;
     RI_REQUIRE(scale > 0.f, "attention_decode_bf16: the scale %g must be positive", (double)scale);
     if (check_common("attention_decode_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width)) return 1;
@@ -1304,12 +1333,12 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
             attn_decode_stream_kernel<DH, false, 8><<<sgrid, 8 * 64, 0, s>>>(                                     \
                 (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, nullptr, nullptr, 0.f, nullptr,            \
                 (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
-                scale_log2, splits, tiled_out, cap_pre, cap_post);                                                \
+                scale_log2, splits, tiled_out, cap_pre, cap_post, slopes, 1.f / scale);                           \
         else                                                                                                      \
             attn_decode_stream_kernel<DH, false, 4><<<sgrid, 4 * 64, 0, s>>>(                                     \
                 (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, nullptr, nullptr, 0.f, nullptr,            \
                 (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
-                scale_log2, splits, tiled_out, cap_pre, cap_post);                                                \
+                scale_log2, splits, tiled_out, cap_pre, cap_post, slopes, 1.f / scale);                           \
         if (splits > 1) launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, -1, splits, tiled_out, s); \
         break;
         switch (head_dim) {
@@ -1327,7 +1356,8 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
     case DH * 16 + CW:                                                                                            \
         attn_decode_mfma_kernel<DH, CW><<<pgrid, CW * 64, 0, s>>>(                                                \
             workspace, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
-            tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, all, cap_pre, cap_post);      \
+            tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, all, cap_pre, cap_post,       \
+            slopes, 1.f / scale);                                                                                 \
         launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, all, tiled_out, s, CW * PAGE);     \
         break;
     switch (head_dim * 16 + DECODE_WAVES / pieces) {
@@ -1376,12 +1406,12 @@ extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const
             attn_decode_stream_kernel<DH, true, 8><<<sgrid, 8 * 64, 0, s>>>(                                      \
                 (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq,             \
                 (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
-                scale_log2, splits, tiled_out, 0.f, 0.f);                                                         \
+                scale_log2, splits, tiled_out, 0.f, 0.f, nullptr, 0.f);                                           \
         else                                                                                                      \
             attn_decode_stream_kernel<DH, true, 4><<<sgrid, 4 * 64, 0, s>>>(                                      \
                 (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq,             \
                 (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
-                scale_log2, splits, tiled_out, 0.f, 0.f);                                                         \
+                scale_log2, splits, tiled_out, 0.f, 0.f, nullptr, 0.f);                                           \
         if (splits > 1) launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, -1, splits, tiled_out, s); \
         break;
         switch (head_dim) {

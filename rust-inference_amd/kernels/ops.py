@@ -52,9 +52,10 @@ _SIGNATURES = {
     "ri_experts_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ri_experts_activate": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
     "ri_attention_prefill_bf16": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
+                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_void_p],
     "ri_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int, c_void_p],
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int,
+                                 c_void_p],
     "ri_attention_decode_fused_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float,
                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                        c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
@@ -541,16 +542,18 @@ def mfma_attention_fits(dtype, head_dim: int, group: int, page_size: int, decode
 
 def attention_prefill_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table, seqs: int, max_new: int,
                            heads: int, kv_heads: int, head_dim: int, window: int | None, scale: float,
-                           softcap: float | None = None) -> torch.Tensor:
+                           softcap: float | None = None, slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Matrix-core attention for any number of new tokens per sequence (bfloat16, pages of 32).  With ``softcap`` a
-    score ``s`` becomes ``softcap * tanh(s / softcap)`` before the softmax."""
+    score ``s`` becomes ``softcap * tanh(s / softcap)`` before the softmax; with ``slopes`` (float32 ``[heads]``) head
+    ``h``'s score at position ``p`` for the key at ``j`` then loses ``slopes[h] * (p - j)``."""
     tokens, stride = qkv.shape
     out = torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
     _call("ri_attention_prefill_bf16", _dev(out, "out"), _dev(qkv, "qkv", torch.bfloat16), stride,
           _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, max_new, heads, kv_heads, head_dim,
-          k_pages.shape[2], int(window or 0), float(scale), float(softcap or 0.0), _stream())
+          k_pages.shape[2], int(window or 0), float(scale), float(softcap or 0.0),
+          _opt(slopes, "slopes", torch.float32, (heads,)), _stream())
     return out
 
 
@@ -569,10 +572,10 @@ def decode_attention_streams(seqs: int, kv_heads: int, max_len: int) -> bool:
 
 def attention_decode_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table, seqs: int, max_len: int,
                           heads: int, kv_heads: int, head_dim: int, window: int | None, scale: float,
-                          tiled_out: bool = False, softcap: float | None = None):
+                          tiled_out: bool = False, softcap: float | None = None, slopes: torch.Tensor | None = None):
     """Matrix-core attention for one new token per sequence; ``max_len`` bounds every sequence's length
     after this step (it sizes the grid and the workspace, not the result).  ``tiled_out``: the result as
-    ``TiledRows`` (at most 64 sequences)."""
+    ``TiledRows`` (at most 64 sequences).  ``softcap`` and ``slopes`` as in ``attention_prefill_bf16``."""
     tokens, stride = qkv.shape
     if tokens != seqs:
         raise ShapeError(f"decode attention takes one token per sequence, got {tokens} tokens for {seqs} sequences")
@@ -585,7 +588,8 @@ def attention_decode_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table
           _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, chunks, heads, kv_heads, head_dim,
-          k_pages.shape[2], int(window or 0), float(scale), float(softcap or 0.0), int(tiled_out), _stream())
+          k_pages.shape[2], int(window or 0), float(scale), float(softcap or 0.0),
+          _opt(slopes, "slopes", torch.float32, (heads,)), int(tiled_out), _stream())
     return out
 
 

@@ -242,8 +242,7 @@ class GroupedQueryAttention(Mixer):
         group = self.heads // self.kv_heads
         cap = self.softcap
         slopes = getattr(self, "slopes", None)
-        if self.v_dim != self.head_dim or slopes is not None:
-            # value heads of their own size, a distance bias: the generic kernel alone takes them
+        if self.v_dim != self.head_dim:          # value heads of their own size: the generic kernel alone takes them
             return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args, cap, slopes)
         if self.rt.invariant:
             # one kernel for prompts and single tokens alike: in the prompt kernel a token's sums run over its
@@ -251,14 +250,14 @@ class GroupedQueryAttention(Mixer):
             # see changes none of its bits); the generic kernel where that one does not take the sizes
             if ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, False):
                 return ops.attention_prefill_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
-                                                  page_table, ctx.B, ctx.max_new, *args, cap)
-            return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args, cap)
+                                                  page_table, ctx.B, ctx.max_new, *args, cap, slopes)
+            return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args, cap, slopes)
         if ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, ctx.is_decode):
             if ctx.is_decode:
                 return ops.attention_decode_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
                                                  page_table, ctx.B, ctx.max_len, *args,
                                                  tiled_out=self.rt.takes_tiled(self.w_o, ctx.B, self.b_o is None),
-                                                 softcap=cap)
+                                                 softcap=cap, slopes=slopes)
             return ops.attention_prefill_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
-                                              page_table, ctx.B, ctx.max_new, *args, cap)
-        return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args, cap)
+                                              page_table, ctx.B, ctx.max_new, *args, cap, slopes)
+        return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args, cap, slopes)

@@ -256,3 +256,92 @@ def test_experts_activation(ops, dtype):
     got = ops.experts_activate(t(gu.reshape(T, -1), dtype), t(dense), ff, limit)
     close(got, want.reshape(T, -1), F32 if dtype == torch.float32 else BF16_OUT)
     assert (f64(got).reshape(T, E, ff)[dense == 0] == 0).all()
+
+
+# ---------------------------------------------------------------- the distance bias on the matrix cores
+def paged_batch(ops, k, v, lens, seed):
+    """Keys and values of several sequences (flat, one after the other) in pages handed out in shuffled order."""
+    G, dk, dv = k.shape[1], k.shape[2], v.shape[2]
+    width = max(-(-n // PAGE) for n in lens) + 1
+    n_pages = sum(-(-n // PAGE) for n in lens) + 2
+    order = np.random.default_rng(seed).permutation(n_pages)
+    table = np.full((len(lens), width), -1, dtype=np.int32)
+    kp = torch.zeros((n_pages, G, PAGE, dk), dtype=torch.bfloat16)
+    vp = torch.zeros((n_pages, G, dv, PAGE), dtype=torch.bfloat16)
+    nxt = at = 0
+    for b, n in enumerate(lens):
+        for p in range(-(-n // PAGE)):
+            table[b, p] = order[nxt]
+            nxt += 1
+        for j in range(n):
+            kp[table[b, j // PAGE], :, j % PAGE] = torch.tensor(k[at + j]).bfloat16()
+            vp[table[b, j // PAGE], :, :, j % PAGE] = torch.tensor(v[at + j]).bfloat16()
+        at += n
+    return guarded(kp.to(DEV)), guarded(vp.to(DEV)), t(table, torch.int32)
+
+
+@pytest.mark.parametrize("form", ["prefill", "decode"])
+@pytest.mark.parametrize("dh, heads, kv_heads, window", [(64, 8, 2, 40), (128, 4, 1, None), (32, 2, 2, 33), (64, 6, 3, 100), (64, 16, 1, 7)])
+def test_the_matrix_core_kernels_take_the_distance_bias(ops, form, dh, heads, kv_heads, window):
+    """bfloat16, heads of 32, 64 and 128, with and without a window: prompts of unequal lengths, and one new token each
+    after them; scores small enough for the bias to decide most weights."""
+    rng = np.random.default_rng(dh + heads)
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dh, "vdim": dh, "scale": 0.05}
+    if window:
+        m["mask"] = {"size": window}
+    lens = [75, 1, 40] if form == "prefill" else [300, 33, 64]
+    T = sum(lens)
+    q, k, v = (bf16_round(rng.normal(size=(T, heads, dh))), bf16_round(rng.normal(size=(T, kv_heads, dh))),
+               bf16_round(rng.normal(size=(T, kv_heads, dh))))
+    kp, vp, table = paged_batch(ops, k, v, lens, dh)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    tok_pos = np.concatenate([np.arange(n) for n in lens])
+    tok_seq = np.repeat(np.arange(len(lens)), lens)
+    want = np.concatenate([P.attention_core(m, q[a:b], k[a:b], v[a:b], np.arange(b - a)).reshape(b - a, -1)
+                           for a, b in zip(cu[:-1], cu[1:])])
+    slopes = t(P.distance_slopes(heads))
+    qkv = t(q.reshape(T, -1), torch.bfloat16)
+    if form == "prefill":
+        got = ops.attention_prefill_bf16(qkv, kp, vp, t(cu, torch.int32), t(tok_pos, torch.int32), table, len(lens), max(lens),
+                                         heads, kv_heads, dh, window, m["scale"], None, slopes)
+        close(got, want, BF16_OUT, "prefill")
+    else:
+        last = cu[1:] - 1                                      # each sequence's last token as its one new token
+        rows = t(q[last].reshape(len(lens), -1), torch.bfloat16)
+        got = ops.attention_decode_bf16(rows, kp, vp, t(np.arange(len(lens) + 1), torch.int32),
+                                        t([n - 1 for n in lens], torch.int32), table, len(lens), max(lens), heads, kv_heads,
+                                        dh, window, m["scale"], slopes=slopes)
+        close(got, want[last], BF16_OUT, "decode")
+    same = ops.attention(qkv, kp, vp, t(tok_pos, torch.int32), t(tok_seq, torch.int32), table, heads, kv_heads, dh, window,
+                         m["scale"], None, slopes)
+    close(same, want, BF16_OUT, "the generic kernel on the same pages")
+
+
+def test_the_matrix_core_kernels_weigh_two_equal_keys_by_their_distance(ops):
+    """Two keys with the same large product with the last query, 1,200 and 3 positions back: without the bias they
+    share the weight, with it the near one has it all, for the one-token kernels and the prompt kernel alike."""
+    rng = np.random.default_rng(4)
+    n, dh, heads = 1300, 64, 2
+    m = {"heads": heads, "kv_heads": 1, "dim": dh, "vdim": dh, "scale": 1.0}
+    k, v, q = rng.normal(size=(n, 1, dh)) * 0.1, rng.normal(size=(n, 1, dh)), rng.normal(size=(n, heads, dh)) * 0.1
+    for j in (n - 1 - 1200, n - 1 - 3):
+        k[j, 0] = 0.0
+        k[j, 0, 9] = 6.0
+    q[-1] = 0.0
+    q[-1, :, 9] = 6.0
+    q, k, v = bf16_round(q), bf16_round(k), bf16_round(v)
+    kp, vp, table = paged_batch(ops, k, v, [n], 1)
+    want = P.attention_core(m, q, k, v, np.arange(n)).reshape(n, -1)
+    near = v[n - 1 - 3, 0]
+    assert np.abs(want[-1, :dh] - near).max() < 1e-3            # head 0's slope is 1/16: 1,197 positions are 75 in the exponent
+    slopes = t(P.distance_slopes(heads))
+    qkv = t(q.reshape(n, -1), torch.bfloat16)
+    whole = ops.attention_prefill_bf16(qkv, kp, vp, t([0, n], torch.int32), t(np.arange(n), torch.int32), table, 1, n, heads, 1,
+                                       dh, None, 1.0, None, slopes)
+    last = ops.attention_decode_bf16(t(q[-1:].reshape(1, -1), torch.bfloat16), kp, vp, t([0, 1], torch.int32),
+                                     t([n - 1], torch.int32), table, 1, n, heads, 1, dh, None, 1.0, slopes=slopes)
+    close(whole, want, BF16_OUT, "prompt")
+    close(last, want[-1:], BF16_OUT, "one token")
+    plain = ops.attention_decode_bf16(t(q[-1:].reshape(1, -1), torch.bfloat16), kp, vp, t([0, 1], torch.int32),
+                                      t([n - 1], torch.int32), table, 1, n, heads, 1, dh, None, 1.0)
+    assert np.abs(f64(plain)[0, :dh] - near).max() > 0.1         # without slopes the far key has half the weight
