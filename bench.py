@@ -2,7 +2,7 @@
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--model 8b|0.6b|1.7b|4b|14b|32b]
-    python bench.py --design zidepel [--size 0.6b|8b] [--layers L]      # another workload: see design_comparison below
+    python bench.py --design zidepel|pisulorn [--size 0.6b|8b] [--layers L]      # another workload: see design_comparison below
 
 The default run has the layer sizes of Qwen3-8B with random weights
 (N(0, 0.02), norm gains 1 + N(0, 0.1), seed 2), a batch of 8 and prompts of 2,048 tokens in a
@@ -208,12 +208,49 @@ def zidepel_like(q, layers, vocab, context):
             "streams": 4, "layers": [rec if i % 4 == 2 else att for i in range(layers)]}
 
 
+def pisulorn_like(q, layers, vocab, context):
+    """A Pisulorn configuration with the layer sizes of a Qwen3 one: the same width, heads and head size, a window of
+    1,024 keys; of every four layers the first has a dense feed-forward half again as wide as Qwen3's, the second and
+    the fourth eight experts of half Qwen3's width of which a token uses two (as many weights in use as the dense
+    one has, four times as many held), and the third is a gated delta rule with as many heads and no feed-forward
+    behind it; four residual streams."""
+    d, h, g, dh, ff = q["hidden_size"], q["num_attention_heads"], q["num_key_value_heads"], q["head_dim"], q["intermediate_size"]
+    mixer = {"heads": h, "kv_heads": g, "dim": dh, "vdim": dh, "scale": dh ** -0.5, "mask": {"size": 1024},
+             "q_temp": {"coef": 0.1, "every": 512}}
+    dense = {"type": "attention", "mlp": {"kind": "dense", "ff": ff * 3 // 2}, "mixer": mixer}
+    moe = {"type": "attention", "mixer": mixer,
+           "mlp": {"kind": "moe", "expert": {"ff": ff // 2, "limit": 7.0}, "router": {"experts": 8, "top": 2}}}
+    rec = {"type": "delta", "mlp": None, "mixer": {"heads": h, "kv_heads": g, "dim": dh, "vdim": dh, "conv": 4}}
+    return {"architecture": "Pisulorn", "vocab": vocab, "width": d, "norm": {"eps": 1e-5}, "streams": 4, "residual_mult": 0.5,
+            "layers": [(dense, moe, rec, moe)[i % 4] for i in range(layers)]}
+
+
 def design_comparison(args) -> int:
-    """`--design zidepel`: prefill and decode of a Zidepel model beside the Qwen3 model of the same layer sizes
-    (random weights, `--layers` layers each, default 8, and a vocabulary of 32,768 for both so that the layers and not
+    """`--design zidepel` or `--design pisulorn`: prefill and decode of a model of that design beside the Qwen3 model
+    of the same layer sizes (and, for Pisulorn, beside the Zidepel model of those sizes, the design closest to it)
+    (random weights, `--layers` layers each, default 8, and a vocabulary of 32,768 for all so that the layers and not
     the output matrix are what is timed).  One JSON line; the default workload and its line are not touched."""
     sizes = {"0.6b": QWEN3_0_6B, "8b": QWEN3_8B}
     layers, vocab, context = args.layers or 8, 32768, args.context
+    if args.design == "pisulorn":
+        out = {"metric": "prefill and decode of the Pisulorn design beside Zidepel and Qwen3 at equal layer sizes", "unit": "tok/s",
+               "n_gpus": 1, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids", "layers": layers,
+               "vocab": vocab, "steps": args.steps, "warmup": args.warmup, "sizes": {}}
+        for size in ([args.size] if args.size else ["0.6b", "8b"]):
+            q = dict(sizes[size], num_hidden_layers=layers, vocab_size=vocab, max_position_embeddings=context,
+                     tie_word_embeddings=False)
+            trio = {}
+            for name, cfg in (("qwen3", q), ("zidepel", zidepel_like(q, layers, vocab, context)),
+                              ("pisulorn", pisulorn_like(q, layers, vocab, context))):
+                b = ShapeBench(f"{name} at Qwen3-{size} layer sizes", cfg, vocab, 11, context, not args.no_graphs)
+                trio[name] = b.measure(args.prompt, (1, 8, 32), args.steps, args.warmup)
+                b.close()
+            out["sizes"][size] = trio
+        first = out["sizes"][next(iter(out["sizes"]))]
+        out["value"], out["higher_is_better"] = first["pisulorn"]["decode_b8"]["tok_s"], True
+        out["vs_zidepel_decode_b8"] = round(first["pisulorn"]["decode_b8"]["tok_s"] / first["zidepel"]["decode_b8"]["tok_s"], 3)
+        print(json.dumps(out))
+        return 0
     out = {"metric": "prefill and decode of the Zidepel design beside Qwen3 at equal layer sizes", "unit": "tok/s",
            "n_gpus": 1, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids", "layers": layers,
            "vocab": vocab, "steps": args.steps, "warmup": args.warmup, "sizes": {}}
@@ -248,7 +285,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the other models")
     ap.add_argument("--no-other-models", action="store_true", help="skip the Qwen3-0.6B and Qwen3-32B points")
     ap.add_argument("--no-graphs", action="store_true", help="launch every kernel of a decode step from the host")
-    ap.add_argument("--design", choices=["zidepel"], default=None,
+    ap.add_argument("--design", choices=["zidepel", "pisulorn"], default=None,
                     help="another workload: this design beside Qwen3 at equal layer sizes (prefill, decode at batch 1, 8, 32)")
     ap.add_argument("--size", choices=["0.6b", "8b"], default=None, help="with --design: one of the two layer sizes only")
     args = ap.parse_args()

@@ -138,9 +138,29 @@ int ri_experts_route(int32_t* ids, float* weights, float* dense, const float* z,
                      int experts, int top, void* stream);
 // The experts' activation on the gate and up branches of all experts side by side: gu [tokens, experts, 2, ff]
 // (gate then up); g = min(gate, limit), u = clamp(up, -limit, limit);
-// out[t, e, i] = dense[t, e] * g * sigmoid(1.702 g) * (u + 1), zero for experts that the token did not choose.
+// out[t, e, i] = dense[t, e] * g * sigmoid(1.702 g) * (u + 1), zero for experts that the token did not choose
+// (dense NULL: every weight 1).
 int ri_experts_activate(void* out, const void* gu, int dtype, const float* dense, int tokens, int experts, int ff,
                         float limit, void* stream);
+
+// Many tokens: the assignments (token t's k-th expert is assignment t * top + k) sorted by expert and, inside an
+// expert, by token.  dest[p]: the row of assignment p; offsets[e]: where expert e's rows begin (experts + 1
+// entries); rank and counts: workspaces of `pairs` and `experts` entries.  ri_experts_gather copies every
+// assignment's token row (bfloat16, dim a multiple of 8) to its place; ri_experts_combine adds a token's rows of y
+// (bfloat16 [pairs, dim]) times the router's weights, in the order chosen, into float32 out [tokens, dim].
+int ri_experts_sort(int32_t* dest, int32_t* offsets, int32_t* rank, int32_t* counts, const int32_t* ids, int pairs,
+                    int experts, void* stream);
+int ri_experts_gather(void* rows, const void* x, const int32_t* dest, int pairs, int top, int dim, void* stream);
+int ri_experts_combine(float* out, const void* y, const int32_t* dest, const float* weights, int tokens, int top, int dim,
+                       void* stream);
+
+// The experts of a few tokens, reading only the rows of the experts chosen (bfloat16): x [tokens, dim]; gu
+// [experts * 2 * ff, dim] (every expert's gate rows, then its up rows); down [dim, experts * ff]; ids and weights
+// [tokens, top] from ri_experts_route; act: workspace [tokens * top, ff] bfloat16; out: float32 [tokens, dim], the
+// weighted sum of the chosen experts' outputs, added in the order chosen.
+int ri_experts_few_tokens(float* out, void* act, const void* x, const void* gu, const void* down, const int32_t* ids,
+                          const float* weights, int tokens, int experts, int top, int ff, int dim, float limit,
+                          void* stream);
 
 // out[i] = max(y[i], 0)^2.
 int ri_relu_squared(void* out, const void* y, int dtype, long total, void* stream);

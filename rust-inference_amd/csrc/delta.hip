@@ -7,7 +7,7 @@
 //     beta = sigmoid(b),   g = exp(-exp(A_log) * softplus(a + dt_bias))               per value head
 //     S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q.
 // Everything after the projections is float32.  ri_delta_prepare makes q, k, v, g and beta of all tokens of a step
-// (one workgroup a token), ri_delta_tails then moves the convolutions' last inputs into the sequences' state, and
+// (a workgroup a token and head), ri_delta_tails then moves the convolutions' last inputs into the sequences' state, and
 // ri_delta_scan walks every sequence's tokens in order.  A token's sums are taken in the same order whatever step
 // or block of tokens it falls into.
 #include "api.h"
@@ -18,7 +18,12 @@
 __device__ __forceinline__ float silu_f(float v) { return v / (1.f + expf(-v)); }
 __device__ __forceinline__ float softplus_f(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 
-// One workgroup a token.  conv[] (dynamic LDS, channels floats) holds the token's activated convolutions.
+// A workgroup takes one token and one unit of its channels: a q or k head (units 0 .. 2 kv_heads - 1), which it
+// norms, or a stretch of DELTA_V_UNIT channels of v.  conv[] (dynamic LDS, max(dim, DELTA_V_UNIT) floats) holds the
+// unit's activated convolutions.  (One workgroup a token walked its thousands of channels in turns of 256, each
+// turn waiting for its own loads: 22 us for a single token.)
+#define DELTA_V_UNIT 256
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 delta_prepare_kernel(float* __restrict__ qkv, float* __restrict__ gates, const T* __restrict__ proj, int row, int q_off,
@@ -27,33 +32,59 @@ delta_prepare_kernel(float* __restrict__ qkv, float* __restrict__ gates, const T
                      const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ cu_seqlens,
                      const int32_t* __restrict__ slots, int heads, int kv_heads, int dim, int vdim) {
     extern __shared__ float conv[];
-    const int t = blockIdx.x, b = tok_seq[t];
+    __shared__ float scratch[16];
+    const int t = blockIdx.x, unit = blockIdx.y, b = tok_seq[t];
     const int i = t - cu_seqlens[b];                          // the token's place among its sequence's new tokens
     const int qk = kv_heads * dim, channels = 2 * qk + heads * vdim;
+    const bool normed = unit < 2 * kv_heads;
+    const int first = normed ? unit * dim : 2 * qk + (unit - 2 * kv_heads) * DELTA_V_UNIT;
+    const int count = normed ? dim : min(DELTA_V_UNIT, channels - first);
     const float* tail = tails + (size_t)slots[b] * (ntaps - 1) * channels;
-    for (int c = threadIdx.x; c < channels; c += blockDim.x) {
-        float y = 0.f;
-        for (int d = ntaps - 1; d >= 0; --d) {                // oldest input first
-            const int at = i - d;
-            const float x = at >= 0 ? to_f32(proj[(size_t)(t - d) * row + q_off + c])
-                                    : tail[(size_t)(ntaps - 1 + at) * channels + c];
-            y += taps[(size_t)c * ntaps + (ntaps - 1 - d)] * x;
+    if (ntaps <= 4) {
+        // the usual few taps: all inputs asked for at once, whatever their place (an address that is not used is
+        // pulled back to one that exists), so that no load waits for another
+        const float* tail_safe = ntaps > 1 ? tail : taps;
+        for (int e = threadIdx.x; e < count; e += blockDim.x) {
+            const int c = first + e;
+            float x[4], w[4];
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const int at = i - d;
+                const float a = to_f32(proj[(size_t)(t - min(d, i)) * row + q_off + c]);
+                const float bb = tail_safe[(size_t)min(max(ntaps - 1 + at, 0), max(ntaps - 2, 0)) * channels + c];
+                x[d] = at >= 0 ? a : bb;
+                w[d] = d < ntaps ? taps[(size_t)c * ntaps + max(ntaps - 1 - d, 0)] : 0.f;
+            }
+            float y = 0.f;
+#pragma unroll
+            for (int d = 3; d >= 0; --d) y += d < ntaps ? w[d] * x[d] : 0.f;           // oldest input first
+            conv[e] = silu_f(y);
         }
-        conv[c] = silu_f(y);
+    } else {
+        for (int e = threadIdx.x; e < count; e += blockDim.x) {
+            const int c = first + e;
+            float y = 0.f;
+            for (int d = ntaps - 1; d >= 0; --d) {                // oldest input first
+                const int at = i - d;
+                const float x = at >= 0 ? to_f32(proj[(size_t)(t - d) * row + q_off + c])
+                                        : tail[(size_t)(ntaps - 1 + at) * channels + c];
+                y += taps[(size_t)c * ntaps + (ntaps - 1 - d)] * x;
+            }
+            conv[e] = silu_f(y);
+        }
     }
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
-    float* out = qkv + (size_t)t * channels;
-    for (int h = wave; h < 2 * kv_heads; h += waves) {        // q heads, then k heads
-        const float* x = conv + (size_t)h * dim;
+    float* out = qkv + (size_t)t * channels + first;
+    if (normed) {                                             // a q head (also times dim^(-1/2)) or a k head
         float ss = 0.f;
-        for (int d = lane; d < dim; d += 64) ss += x[d] * x[d];
-        ss = wave_sum(ss);
-        const float f = (h < kv_heads ? rsqrtf((float)dim) : 1.f) / sqrtf(ss + 1e-6f);
-        for (int d = lane; d < dim; d += 64) out[(size_t)h * dim + d] = x[d] * f;
+        for (int e = threadIdx.x; e < count; e += blockDim.x) ss += conv[e] * conv[e];
+        ss = block_sum(ss, scratch);
+        const float f = (unit < kv_heads ? rsqrtf((float)dim) : 1.f) / sqrtf(ss + 1e-6f);
+        for (int e = threadIdx.x; e < count; e += blockDim.x) out[e] = conv[e] * f;
+    } else {
+        for (int e = threadIdx.x; e < count; e += blockDim.x) out[e] = conv[e];
     }
-    for (int c = 2 * qk + threadIdx.x; c < channels; c += blockDim.x) out[c] = conv[c];
-    if (threadIdx.x < heads) {
+    if (unit == 0 && threadIdx.x < heads) {
         const int h = threadIdx.x;
         const float a = ab[(size_t)t * 2 * heads + h], bb = ab[(size_t)t * 2 * heads + heads + h];
         gates[(size_t)t * 2 * heads + h] = expf(-expf(a_log[h]) * softplus_f(a + dt_bias[h]));
@@ -77,6 +108,15 @@ delta_tails_kernel(float* __restrict__ tails, const T* __restrict__ proj, int ro
         v[r] = at < keep ? tail[(size_t)at * channels + c] : to_f32(proj[(size_t)(t0 + at - keep) * row + q_off + c]);
     }
     for (int r = 0; r < keep; ++r) tail[(size_t)r * channels + c] = v[r];
+}
+
+// The sum over the four lanes of a quad, in each of them, by two quad permutations of the vector unit's own data
+// path (DPP): [1, 0, 3, 2] then [2, 3, 0, 1].  A shuffle goes through the LDS crossbar instead, and the walk waits
+// for four of them in a row at every token.
+__device__ __forceinline__ float quad_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));
+    return v;
 }
 
 // The walk.  A workgroup owns one (sequence, value head) and 64 columns of its state: 64 columns x 4 slices of
@@ -166,26 +206,26 @@ delta_scan_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
         fetch(more ? first + DELTA_BLOCK : first);            // (always issued: no load in a branch)
         const DeltaLds<RPT>& l = lds[cur];
         const int count = min(DELTA_BLOCK, n - first);
+#pragma unroll 2
         for (int tk = 0; tk < count; ++tk) {
             const float g = l.g[tk], beta = l.beta[tk];
-            float kk[RPT], dot = 0.f;
+            // four partial sums each: a single one would be a chain of RPT dependent additions
+            float kk[RPT], d4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
                 kk[i] = l.k[tk][r][i];
                 S[i] *= g;
-                dot += S[i] * kk[i];
+                d4[i & 3] += S[i] * kk[i];
             }
-            dot += __shfl_xor(dot, 1, RI_WAVE);
-            dot += __shfl_xor(dot, 2, RI_WAVE);
+            const float dot = quad_sum((d4[0] + d4[1]) + (d4[2] + d4[3]));
             const float u = beta * (l.v[tk][tid >> 2] - dot);
-            float o = 0.f;
+            float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
                 S[i] += kk[i] * u;
-                o += S[i] * l.q[tk][r][i];
+                o4[i & 3] += S[i] * l.q[tk][r][i];
             }
-            o += __shfl_xor(o, 1, RI_WAVE);
-            o += __shfl_xor(o, 2, RI_WAVE);
+            const float o = quad_sum((o4[0] + o4[1]) + (o4[2] + o4[3]));
             if (r == 0 && has_col) out[(size_t)(t0 + first + tk) * heads * vdim + (size_t)h * vdim + col] = o;
         }
         stage(lds[cur ^ 1]);
@@ -211,16 +251,19 @@ extern "C" int ri_delta_prepare(float* qkv, float* gates, const void* proj, int 
     RI_REQUIRE(ntaps >= 1 && ntaps <= DELTA_MAX_TAPS, "delta_prepare: %d taps, the kernels take 1 to %d", ntaps, DELTA_MAX_TAPS);
     const long channels = 2L * kv_heads * dim + (long)heads * vdim;
     RI_REQUIRE(q_off >= 0 && q_off + channels <= row, "delta_prepare: %ld channels at column %d of rows of %d", channels, q_off, row);
-    RI_REQUIRE(channels * 4 <= 64 * 1024, "delta_prepare: %ld channels exceed the workgroup's memory", channels);
+    RI_REQUIRE(dim <= 8192, "delta_prepare: heads of %d exceed the workgroup's memory", dim);
     RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "delta_prepare: dtype %d", act_dtype);
     hipStream_t s = (hipStream_t)stream;
-    const size_t shared = (size_t)channels * sizeof(float);
+    const size_t shared = (size_t)(dim > DELTA_V_UNIT ? dim : DELTA_V_UNIT) * sizeof(float);
+    const int units = 2 * kv_heads + (heads * vdim + DELTA_V_UNIT - 1) / DELTA_V_UNIT;
+    RI_REQUIRE(units <= 65535, "delta_prepare: %d units of channels exceed one launch", units);
+    const dim3 pgrid(tokens, units);
     if (act_dtype == RI_F32) {
-        delta_prepare_kernel<float><<<tokens, 256, shared, s>>>(qkv, gates, (const float*)proj, row, q_off, taps, ntaps, tails,
+        delta_prepare_kernel<float><<<pgrid, 256, shared, s>>>(qkv, gates, (const float*)proj, row, q_off, taps, ntaps, tails,
                                                                ab, a_log, dt_bias, tok_seq, cu_seqlens, slots, heads,
                                                                kv_heads, dim, vdim);
     } else {
-        delta_prepare_kernel<bf16_t><<<tokens, 256, shared, s>>>(qkv, gates, (const bf16_t*)proj, row, q_off, taps, ntaps,
+        delta_prepare_kernel<bf16_t><<<pgrid, 256, shared, s>>>(qkv, gates, (const bf16_t*)proj, row, q_off, taps, ntaps,
                                                                 tails, ab, a_log, dt_bias, tok_seq, cu_seqlens, slots,
                                                                 heads, kv_heads, dim, vdim);
     }

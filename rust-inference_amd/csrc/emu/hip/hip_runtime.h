@@ -158,6 +158,15 @@ static inline int emu_readfirstlane(int v) {
     const uint64_t live = emu::wave_gather(&v, sizeof(int), all);
     return all[__builtin_ctzll(live)];
 }
+// v_mov_b32 with a DPP quad permutation (control 0x00 .. 0xFF: lane q of every four takes the value of lane
+// (control >> 2q) & 3 of the same four); all rows and banks enabled.
+static inline int emu_mov_dpp_quad(int v, int control) {
+    int all[64];
+    emu::wave_gather(&v, sizeof(int), all);
+    const int lane = emu::self->lane;
+    return all[(lane & ~3) | ((control >> (2 * (lane & 3))) & 3)];
+}
+#define __builtin_amdgcn_mov_dpp(v, control, row_mask, bank_mask, bound_ctrl) emu_mov_dpp_quad((v), (control))
 #define __builtin_amdgcn_readlane(v, l) emu_readlane((int)(v), (l))
 #define __builtin_amdgcn_readfirstlane(v) emu_readfirstlane((int)(v))
 // The lanes of a wavefront run in step on the GPU, so what one lane has written to LDS another lane reads

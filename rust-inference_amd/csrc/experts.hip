@@ -47,7 +47,7 @@ __global__ void __launch_bounds__(256)
 experts_activate_kernel(T* __restrict__ out, const T* __restrict__ gu, const float* __restrict__ dense, int experts, int ff,
                         float limit) {
     const int t = blockIdx.x, e = blockIdx.y;
-    const float w = dense[(size_t)t * experts + e];
+    const float w = dense ? dense[(size_t)t * experts + e] : 1.f;        // no weights: every row is of its expert
     T* o = out + ((size_t)t * experts + e) * ff;
     const T* g = gu + ((size_t)t * experts + e) * 2 * ff;
     for (int i = threadIdx.x; i < ff; i += blockDim.x) {
@@ -59,6 +59,179 @@ experts_activate_kernel(T* __restrict__ out, const T* __restrict__ gu, const flo
         }
         from_f32(o + i, v);
     }
+}
+
+// ---- a few tokens: only the chosen experts' rows are read
+// One wavefront an (assignment, row i): the gate row i and the up row i of the assignment's expert against the
+// token's row, 16 bytes a lane at a time, then the activation times the router's weight.  gu: [experts, 2, ff, dim]
+// rows (gate then up); act: [tokens * top, ff].
+__global__ void __launch_bounds__(256)
+experts_gate_up_rows_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__ x, const bf16_t* __restrict__ gu,
+                            const int32_t* __restrict__ ids, const float* __restrict__ weights, int top, int ff, int dim,
+                            float limit) {
+    const int lane = threadIdx.x & 63, i = blockIdx.x * 4 + (threadIdx.x >> 6), pair = blockIdx.y;
+    if (i >= ff) return;                                      // (whole wavefronts)
+    const int e = ids[pair];
+    const bf16_t* xr = x + (size_t)(pair / top) * dim;
+    const bf16_t* gr = gu + ((size_t)e * 2 * ff + i) * dim;
+    const bf16_t* ur = gr + (size_t)ff * dim;
+    float g = 0.f, u = 0.f;
+    for (int c = lane * 8; c < dim; c += 512) {
+        const uint4 a = load_stream16(gr + c), b = load_stream16(ur + c), v = *reinterpret_cast<const uint4*>(xr + c);
+        const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w}, vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float x0 = __uint_as_float(vw[k] << 16), x1 = __uint_as_float(vw[k] & 0xFFFF0000u);
+            g += __uint_as_float(aw[k] << 16) * x0 + __uint_as_float(aw[k] & 0xFFFF0000u) * x1;
+            u += __uint_as_float(bw[k] << 16) * x0 + __uint_as_float(bw[k] & 0xFFFF0000u) * x1;
+        }
+    }
+    g = wave_sum(g);
+    u = wave_sum(u);
+    if (lane == 0) {
+        // the products' results pass through bfloat16, as they do where the products are kernels of their own
+        const float gg = fminf(bf16_to_f32(f32_to_bf16(g)), limit);
+        const float uu = fminf(fmaxf(bf16_to_f32(f32_to_bf16(u)), -limit), limit);
+        act[(size_t)pair * ff + i] = f32_to_bf16(weights[pair] * (gg / (1.f + expf(-1.702f * gg)) * (uu + 1.f)));
+    }
+}
+
+// One wavefront an output row n of a token: the sum over the token's chosen experts, in the order chosen, of the
+// expert's down row n against the assignment's activations.  down: [dim, experts * ff] (the experts side by side
+// along a row); out: float32 [tokens, dim].
+__global__ void __launch_bounds__(256)
+experts_down_rows_kernel(float* __restrict__ out, const bf16_t* __restrict__ act, const bf16_t* __restrict__ down,
+                         const int32_t* __restrict__ ids, int top, int ff, int dim, int experts) {
+    const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6), t = blockIdx.y;
+    if (n >= dim) return;
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) {
+        const int pair = t * top + k;
+        const bf16_t* wr = down + (size_t)n * experts * ff + (size_t)ids[pair] * ff;
+        const bf16_t* ar = act + (size_t)pair * ff;
+        for (int c = lane * 8; c < ff; c += 512) {
+            const uint4 a = load_stream16(wr + c), v = *reinterpret_cast<const uint4*>(ar + c);
+            const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc += __uint_as_float(aw[j] << 16) * __uint_as_float(vw[j] << 16)
+                     + __uint_as_float(aw[j] & 0xFFFF0000u) * __uint_as_float(vw[j] & 0xFFFF0000u);
+        }
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) out[(size_t)t * dim + n] = acc;
+}
+
+extern "C" int ri_experts_few_tokens(float* out, void* act, const void* x, const void* gu, const void* down,
+                                     const int32_t* ids, const float* weights, int tokens, int experts, int top, int ff,
+                                     int dim, float limit, void* stream) {
+    RI_REQUIRE(tokens > 0 && experts >= 1 && top >= 1 && top <= experts, "experts_few_tokens: %d tokens, %d of %d experts",
+               tokens, top, experts);
+    RI_REQUIRE(ff >= 8 && ff % 8 == 0 && dim >= 8 && dim % 8 == 0, "experts_few_tokens: sizes %d and %d must be multiples of 8", ff, dim);
+    RI_REQUIRE((long)tokens * top <= 65535 && tokens <= 65535, "experts_few_tokens: %d tokens exceed one launch", tokens);
+    hipStream_t s = (hipStream_t)stream;
+    experts_gate_up_rows_kernel<<<dim3((ff + 3) / 4, tokens * top), 256, 0, s>>>(
+        (bf16_t*)act, (const bf16_t*)x, (const bf16_t*)gu, ids, weights, top, ff, dim, limit);
+    RI_LAUNCH_CHECK("experts_few_tokens (gate and up)");
+    experts_down_rows_kernel<<<dim3((dim + 3) / 4, tokens), 256, 0, s>>>(out, (const bf16_t*)act, (const bf16_t*)down, ids,
+                                                                       top, ff, dim, experts);
+    RI_LAUNCH_CHECK("experts_few_tokens (down)");
+    return 0;
+}
+
+// ---- many tokens: the assignments sorted by expert, so that every expert's tokens are rows side by side
+// One workgroup an expert: it walks all assignments in order and numbers its own, so that the order inside an
+// expert is the order of the tokens whatever ran first.
+__global__ void __launch_bounds__(256)
+experts_rank_kernel(int32_t* __restrict__ rank, int32_t* __restrict__ counts, const int32_t* __restrict__ ids, int pairs) {
+    __shared__ int wave_count[4];
+    const int e = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int before = 0;
+    for (int base = 0; base < pairs; base += 256) {
+        const int p = base + threadIdx.x;
+        const bool mine = p < pairs && ids[p] == e;
+        const unsigned long long votes = __ballot(mine);
+        if (lane == 0) wave_count[wave] = __builtin_popcountll(votes);
+        __syncthreads();
+        int ahead = __builtin_popcountll(votes & ((1ull << lane) - 1ull)), all = 0;
+        for (int w = 0; w < 4; ++w) {
+            if (w < wave) ahead += wave_count[w];
+            all += wave_count[w];
+        }
+        if (mine) rank[p] = before + ahead;
+        before += all;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) counts[e] = before;
+}
+
+// offsets[e]: where expert e's rows begin (offsets[experts]: the number of assignments); dest[p]: the row of
+// assignment p.  One workgroup.
+__global__ void __launch_bounds__(256)
+experts_place_kernel(int32_t* __restrict__ dest, int32_t* __restrict__ offsets, const int32_t* __restrict__ rank,
+                     const int32_t* __restrict__ counts, const int32_t* __restrict__ ids, int pairs, int experts) {
+    __shared__ int start[EXPERTS_MAX + 1];
+    if (threadIdx.x == 0) {
+        int at = 0;
+        for (int e = 0; e < experts; ++e) {
+            start[e] = at;
+            at += counts[e];
+        }
+        start[experts] = at;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e <= experts; e += blockDim.x) offsets[e] = start[e];
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) dest[p] = start[ids[p]] + rank[p];
+}
+
+// rows[dest[p], :] = x[p / top, :], 16 bytes a thread at a time (dim a multiple of 8 bfloat16).
+__global__ void __launch_bounds__(256)
+experts_gather_kernel(bf16_t* __restrict__ rows, const bf16_t* __restrict__ x, const int32_t* __restrict__ dest, int top,
+                      int dim) {
+    const int p = blockIdx.x;
+    const uint4* from = reinterpret_cast<const uint4*>(x + (size_t)(p / top) * dim);
+    uint4* to = reinterpret_cast<uint4*>(rows + (size_t)dest[p] * dim);
+    for (int c = threadIdx.x; c < dim / 8; c += blockDim.x) to[c] = from[c];
+}
+
+// out[t, :] = sum over the token's assignments k, in order, of weights[t, k] * y[dest[t * top + k], :], in float32.
+__global__ void __launch_bounds__(256)
+experts_combine_kernel(float* __restrict__ out, const bf16_t* __restrict__ y, const int32_t* __restrict__ dest,
+                       const float* __restrict__ weights, int top, int dim) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x; c < dim; c += blockDim.x) {
+        float acc = 0.f;
+        for (int k = 0; k < top; ++k)
+            acc += weights[(size_t)t * top + k] * bf16_to_f32(y[(size_t)dest[(size_t)t * top + k] * dim + c]);
+        out[(size_t)t * dim + c] = acc;
+    }
+}
+
+extern "C" int ri_experts_sort(int32_t* dest, int32_t* offsets, int32_t* rank, int32_t* counts, const int32_t* ids,
+                               int pairs, int experts, void* stream) {
+    RI_REQUIRE(pairs > 0 && experts >= 1 && experts <= EXPERTS_MAX, "experts_sort: %d assignments to %d experts", pairs, experts);
+    hipStream_t s = (hipStream_t)stream;
+    experts_rank_kernel<<<experts, 256, 0, s>>>(rank, counts, ids, pairs);
+    RI_LAUNCH_CHECK("experts_sort (rank)");
+    experts_place_kernel<<<1, 256, 0, s>>>(dest, offsets, rank, counts, ids, pairs, experts);
+    RI_LAUNCH_CHECK("experts_sort (place)");
+    return 0;
+}
+
+extern "C" int ri_experts_gather(void* rows, const void* x, const int32_t* dest, int pairs, int top, int dim, void* stream) {
+    RI_REQUIRE(pairs > 0 && top >= 1 && pairs % top == 0 && dim >= 8 && dim % 8 == 0,
+               "experts_gather: %d assignments, %d a token, rows of %d", pairs, top, dim);
+    experts_gather_kernel<<<pairs, 256, 0, (hipStream_t)stream>>>((bf16_t*)rows, (const bf16_t*)x, dest, top, dim);
+    RI_LAUNCH_CHECK("experts_gather");
+    return 0;
+}
+
+extern "C" int ri_experts_combine(float* out, const void* y, const int32_t* dest, const float* weights, int tokens, int top,
+                                  int dim, void* stream) {
+    RI_REQUIRE(tokens > 0 && top >= 1 && dim >= 1, "experts_combine: %d tokens, %d a token, rows of %d", tokens, top, dim);
+    experts_combine_kernel<<<tokens, 256, 0, (hipStream_t)stream>>>(out, (const bf16_t*)y, dest, weights, top, dim);
+    RI_LAUNCH_CHECK("experts_combine");
+    return 0;
 }
 
 extern "C" int ri_experts_route(int32_t* ids, float* weights, float* dense, const float* z, const float* correction,

@@ -51,6 +51,11 @@ _SIGNATURES = {
                       c_void_p],
     "ri_experts_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ri_experts_activate": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+    "ri_experts_sort": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "ri_experts_gather": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ri_experts_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ri_experts_few_tokens": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                              c_int, c_float, c_void_p],
     "ri_attention_prefill_bf16": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_void_p],
     "ri_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -518,15 +523,73 @@ def experts_route(z: torch.Tensor, correction: torch.Tensor, top: int):
     return ids, weights, dense
 
 
-def experts_activate(gu: torch.Tensor, dense: torch.Tensor, ff: int, limit: float) -> torch.Tensor:
+def experts_sort(ids: torch.Tensor, experts: int):
+    """The assignments ``ids [T, top]`` sorted by expert and, inside an expert, by token: ``dest [T * top]`` (the row
+    of assignment ``t * top + k``) and ``offsets [experts + 1]`` (where every expert's rows begin), int32."""
+    pairs = ids.numel()
+    dest = torch.empty((pairs,), dtype=torch.int32, device=ids.device)
+    rank = torch.empty((pairs,), dtype=torch.int32, device=ids.device)
+    offsets = torch.empty((experts + 1,), dtype=torch.int32, device=ids.device)
+    counts = torch.empty((experts,), dtype=torch.int32, device=ids.device)
+    _call("ri_experts_sort", _dev(dest, "dest"), _dev(offsets, "offsets"), _dev(rank, "rank"), _dev(counts, "counts"),
+          _dev(ids, "ids", torch.int32), pairs, experts, _stream())
+    return dest, offsets
+
+
+def experts_gather(x: torch.Tensor, dest: torch.Tensor, top: int) -> torch.Tensor:
+    """``rows[dest[t * top + k]] = x[t]``: every assignment's token row at its place among its expert's rows."""
+    tokens, dim = x.shape
+    rows = torch.empty((tokens * top, dim), dtype=x.dtype, device=x.device)
+    _call("ri_experts_gather", _dev(rows, "rows"), _dev(x, "x", torch.bfloat16), _dev(dest, "dest", torch.int32, (tokens * top,)),
+          tokens * top, top, dim, _stream())
+    return rows
+
+
+def experts_combine(y: torch.Tensor, dest: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+    """float32 ``out[t] = sum_k weights[t, k] * y[dest[t * top + k]]``, the sum in the order chosen."""
+    tokens, top = weights.shape
+    dim = y.shape[1]
+    out = torch.empty((tokens, dim), dtype=torch.float32, device=y.device)
+    _call("ri_experts_combine", _dev(out, "out"), _dev(y, "y", torch.bfloat16, (tokens * top, dim)),
+          _dev(dest, "dest", torch.int32, (tokens * top,)), _dev(weights, "weights", torch.float32), tokens, top, dim, _stream())
+    return out
+
+
+def experts_activate(gu: torch.Tensor, dense, ff: int, limit: float) -> torch.Tensor:
     """``dense[t, e] * g sigmoid(1.702 g) (u + 1)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``
-    for ``gu [T, E * 2 * ff]`` (every expert's gate then up); ``[T, E * ff]``, zero for experts not chosen."""
+    for ``gu [T, E * 2 * ff]`` (every expert's gate then up); ``[T, E * ff]``, zero for experts not chosen.  ``dense``
+    None: rows of one expert each (``gu [T, 2 * ff]``), every weight 1."""
+    if dense is None:
+        tokens = gu.shape[0]
+        out = torch.empty((tokens, ff), dtype=gu.dtype, device=gu.device)
+        if tuple(gu.shape) != (tokens, 2 * ff):
+            raise ShapeError(f"gate|up rows are {list(gu.shape)} for experts of {ff}")
+        _call("ri_experts_activate", _dev(out, "out"), _dev(gu, "gu"), code(gu.dtype), None, tokens, 1, ff, float(limit), _stream())
+        return out
     tokens, experts = dense.shape
     if tuple(gu.shape) != (tokens, experts * 2 * ff):
         raise ShapeError(f"gate|up rows are {list(gu.shape)} for {experts} experts of {ff}")
     out = torch.empty((tokens, experts * ff), dtype=gu.dtype, device=gu.device)
     _call("ri_experts_activate", _dev(out, "out"), _dev(gu, "gu"), code(gu.dtype), _dev(dense, "dense", torch.float32),
           tokens, experts, ff, float(limit), _stream())
+    return out
+
+
+def experts_few_tokens(x, gate_up, down, ids, weights, ff: int, limit: float) -> torch.Tensor:
+    """The weighted sum of the chosen experts' outputs for a few tokens, reading only the chosen experts' rows
+    (bfloat16): ``x [T, dim]``, ``gate_up [E * 2 * ff, dim]``, ``down [dim, E * ff]``, ``ids`` and ``weights``
+    ``[T, top]`` from ``experts_route``; float32 ``[T, dim]``."""
+    tokens, dim = x.shape
+    top = ids.shape[1]
+    experts = gate_up.shape[0] // (2 * ff)
+    if tuple(gate_up.shape) != (experts * 2 * ff, dim) or tuple(down.shape) != (dim, experts * ff):
+        raise ShapeError(f"experts' matrices {list(gate_up.shape)} and {list(down.shape)} for rows of {dim} and experts of {ff}")
+    out = torch.empty((tokens, dim), dtype=torch.float32, device=x.device)
+    act = torch.empty((tokens * top, ff), dtype=torch.bfloat16, device=x.device)
+    _call("ri_experts_few_tokens", _dev(out, "out"), _dev(act, "act"), _dev(x, "x", torch.bfloat16),
+          _dev(gate_up, "gate_up", torch.bfloat16), _dev(down, "down", torch.bfloat16),
+          _dev(ids, "ids", torch.int32, (tokens, top)), _dev(weights, "weights", torch.float32, (tokens, top)),
+          tokens, experts, top, ff, dim, float(limit), _stream())
     return out
 
 

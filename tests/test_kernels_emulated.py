@@ -59,6 +59,8 @@ PYTEST = ["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider"]
 KERNEL_TESTS, SMALL_MACHINE = os.path.join(HERE, "test_kernels_gpu.py"), os.path.join(HERE, "small_machine_kernels.py")
 SAMPLER_TESTS = os.path.join(HERE, "test_sampling_gpu.py")
 ZIDEPEL_TESTS = os.path.join(HERE, "test_zidepel_kernels_gpu.py")
+PISULORN_TESTS = os.path.join(HERE, "test_pisulorn_kernels_gpu.py")
+PISULORN_SELECT = "not two_equal_keys"          # not the 1,300 keys on the emulated matrix cores (minutes)
 SAMPLER_SELECT = "(same_token_as_the_plain_sampler or top_p_drops) and not large"     # not the 151,936 entries, not the engine
 
 
@@ -78,6 +80,7 @@ def runs():
         "one unit": _start([*PYTEST, *_workers(2), SMALL_MACHINE, KERNEL_TESTS, "-k", ONE_UNIT], {"RI_EMU_COMPUTE_UNITS": "1"}),
         "sampler": _start([*PYTEST, *_workers(2), SAMPLER_TESTS, "-k", SAMPLER_SELECT]),
         "zidepel": _start([*PYTEST, *_workers(2), ZIDEPEL_TESTS]),
+        "pisulorn": _start([*PYTEST, *_workers(2), PISULORN_TESTS, "-k", PISULORN_SELECT]),
     }
     done = {}
     try:
@@ -112,6 +115,13 @@ def test_the_kernels_of_the_zidepel_design_pass_on_the_cpu_build_between_guard_p
     temperature and cache write, capped attention (generic and on the emulated matrix cores), the gated linear
     recurrence, the squared ReLU."""
     _passed(runs["zidepel"])
+
+
+def test_the_kernels_of_the_pisulorn_design_pass_on_the_cpu_build_between_guard_pages(runs):
+    """tests/test_pisulorn_kernels_gpu.py: the distance bias and the window (generic and on the emulated matrix
+    cores), the short convolutions with their tails, the gated delta rule's walk, the router, the experts of a few
+    tokens and the sort of many, the tanh form of GELU."""
+    _passed(runs["pisulorn"])
 
 
 @pytest.mark.parametrize("units, tests", [("sixteen units", 7), ("one unit", 61)])

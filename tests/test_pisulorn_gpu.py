@@ -249,6 +249,18 @@ def test_long_decoding_from_the_first_tokens(folders, name, dtype_name):
     against_plain(folders[name], got, reqs, dtype_name, "long decoding")
 
 
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_the_three_ways_through_the_experts_agree(folders, name, dtype_name):
+    """A prompt of 330 tokens (its tokens sorted by expert), the same in portions of 100 (all experts for all tokens)
+    and its last tokens one by one (only the chosen experts' rows are read), with a second request beside it."""
+    reqs = requests_for(name, [330, 290], 9)
+    model = loaded(folders, name, dtype_name)
+    for what, steps in (("whole", plans.whole(reqs)), ("portions of 100", in_portions(reqs, [100])),
+                        ("a batch, then one by one", plans.unequal_batches([{rid: (toks, len(toks) - 6) for rid, toks in reqs.items()}]))):
+        against_plain(folders[name], replay(model, steps), reqs, dtype_name, what)
+
+
 # ---------------------------------------------------------------- a window's edge, made to show
 W_EDGE = {"architecture": "Pisulorn", "vocab": 64, "width": 32, "norm": {"eps": 1e-5},
           "layers": [attention(2, 1, 16, 16, 1.0, 37, None, None)]}

@@ -345,3 +345,55 @@ def test_the_matrix_core_kernels_weigh_two_equal_keys_by_their_distance(ops):
     plain = ops.attention_decode_bf16(t(q[-1:].reshape(1, -1), torch.bfloat16), kp, vp, t([0, 1], torch.int32),
                                       t([n - 1], torch.int32), table, 1, n, heads, 1, dh, None, 1.0)
     assert np.abs(f64(plain)[0, :dh] - near).max() > 0.1         # without slopes the far key has half the weight
+
+
+# ---------------------------------------------------------------- the experts of a few tokens, and of many
+def experts_case(rng, T, E, top, ff, dim, limit):
+    x = bf16_round(rng.normal(size=(T, dim)))
+    w = {"m.router": bf16_round(rng.normal(size=(E, dim)) * 0.3), "m.correction": rng.normal(size=E) * 0.2}
+    for e in range(E):
+        w[f"m.e{e}.gate"] = bf16_round(rng.normal(size=(ff, dim)) * 0.2)
+        w[f"m.e{e}.up"] = bf16_round(rng.normal(size=(ff, dim)) * 0.2)
+        w[f"m.e{e}.down"] = bf16_round(rng.normal(size=(dim, ff)) * 0.2)
+    mlp = {"kind": "moe", "expert": {"ff": ff, "limit": limit}, "router": {"experts": E, "top": top}}
+    gate_up = np.concatenate([np.concatenate([w[f"m.e{e}.gate"], w[f"m.e{e}.up"]]) for e in range(E)])
+    down = np.concatenate([w[f"m.e{e}.down"] for e in range(E)], 1)
+    return x, w, mlp, gate_up, down
+
+
+@pytest.mark.parametrize("T, E, top, ff, dim", [(1, 8, 3, 24, 40), (5, 4, 1, 520, 72), (8, 6, 5, 16, 1032), (3, 3, 2, 8, 8)])
+def test_the_experts_of_a_few_tokens(ops, T, E, top, ff, dim):
+    rng = np.random.default_rng(T + E)
+    x, w, mlp, gate_up, down = experts_case(rng, T, E, top, ff, dim, 0.9)
+    want = P.moe_ff(mlp, w, "m.", x)
+    ids, weights, _ = ops.experts_route(t(x @ w["m.router"].T), t(w["m.correction"]), top)
+    got = ops.experts_few_tokens(t(x, torch.bfloat16), t(gate_up, torch.bfloat16), t(down, torch.bfloat16), ids, weights, ff, 0.9)
+    close(got, want, BF16_OUT)
+
+
+@pytest.mark.parametrize("T, E, top, dim", [(300, 8, 3, 40), (70, 5, 1, 16), (9, 3, 3, 8), (1, 70, 4, 24), (520, 2, 1, 8)])
+def test_the_assignments_sorted_by_expert(ops, T, E, top, dim):
+    rng = np.random.default_rng(T)
+    ids = np.stack([rng.permutation(E)[:top] for _ in range(T)]).astype(np.int32)
+    dest, offsets = ops.experts_sort(t(ids, torch.int32), E)
+    flat = ids.reshape(-1)
+    order = np.argsort(flat, kind="stable")                   # by expert, inside an expert by token
+    want_dest = np.empty_like(order)
+    want_dest[order] = np.arange(len(order))
+    assert np.array_equal(f64(dest).astype(int), want_dest)
+    assert np.array_equal(f64(offsets).astype(int), np.concatenate([[0], np.cumsum(np.bincount(flat, minlength=E))]))
+    x = bf16_round(rng.normal(size=(T, dim)))
+    rows = ops.experts_gather(t(x, torch.bfloat16), dest, top)
+    assert np.array_equal(f64(rows)[want_dest], np.repeat(x, top, 0))
+    weights = rng.uniform(0.1, 1, size=(T, top))
+    y = bf16_round(rng.normal(size=(T * top, dim)))
+    got = ops.experts_combine(t(y, torch.bfloat16), dest, t(weights))
+    close(got, (weights[:, :, None] * y[want_dest].reshape(T, top, dim)).sum(1), F32)
+
+
+def test_an_experts_rows_activated_without_weights(ops):
+    rng = np.random.default_rng(8)
+    gu = rng.normal(size=(7, 2, 20)) * 2
+    g, u = np.minimum(gu[:, 0], 1.1), np.clip(gu[:, 1], -1.1, 1.1)
+    got = ops.experts_activate(t(gu.reshape(7, -1)), None, 20, 1.1)
+    close(got, g * P.sigmoid(1.702 * g) * (u + 1.0), F32)
