@@ -64,8 +64,8 @@ class BiasedAttentionSizes:
             raise ConfigError(f"{where}: an attention mixer needs 'scale'")
         dim = whole(m["dim"], where + ".dim", 1)
         window = None
-        if m.get("mask") is not None:
-            window = whole(_section(m, "mask", where).get("size"), where + ".mask.size", 1)
+        if m.get("mask") is not None and _section(m, "mask", where).get("size") is not None:
+            window = whole(m["mask"]["size"], where + ".mask.size", 1)
         coef, every = None, 1
         if m.get("q_temp") is not None:
             qt = _section(m, "q_temp", where)
