@@ -130,6 +130,15 @@ int ri_delta_max_dim();
 int ri_delta_scan(float* out, const float* qkv, const float* gates, float* state, const int32_t* cu_seqlens,
                   const int32_t* slots, int seqs, int tokens, int heads, int kv_heads, int dim, int vdim, void* stream);
 
+// One new token a sequence (token b is sequence b's; cu_seqlens is 0, 1, .., seqs): ri_delta_prepare, ri_delta_scan, the
+// per-head RMS norm over vdim with `gain` and the gate silu(g) (read from proj rows at column g_off) in one kernel, then
+// the tails moved on; out of act_dtype [seqs, heads * vdim].  ri_delta_step_fits: whether it takes these head sizes.
+int ri_delta_step_fits(int dim, int vdim);
+int ri_delta_step(void* out, const void* proj, int act_dtype, int row, int q_off, int g_off, const float* taps, int ntaps,
+                  float* tails, const float* ab, const float* a_log, const float* dt_bias, float* state,
+                  const int32_t* cu_seqlens, const int32_t* slots, const float* gain, float eps, int seqs, int heads,
+                  int kv_heads, int dim, int vdim, void* stream);
+
 // A mixture of experts' router.  z: float32 [tokens, experts] router logits; s = sigmoid(z); the `top` experts with
 // the largest s + correction (the lower index on a tie) are chosen; their weights are their s divided by the sum of
 // the chosen s (+ 1e-20).  ids: int32 [tokens, top] in the order chosen; weights: float32 [tokens, top]; dense:

@@ -239,6 +239,135 @@ delta_scan_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
     }
 }
 
+// One new token a sequence: the convolutions, the unit norms, the gates, the step on the state, the per-head norm
+// and the output gate in one kernel.  A workgroup owns one (sequence, head): `cols` columns (vdim rounded up to a power
+// of two, 32 at least) x 256 / cols slices of rows, a thread RPT rows of one column in registers; consecutive lanes hold
+// consecutive columns, so the state streams in and out in whole lines.  The sums over rows meet through LDS, slice after
+// slice.  The convolutions' tails are read here and moved on by delta_tails_kernel afterwards (the heads that share a
+// q/k head all read its tail).
+template <typename T, int RPT>
+__global__ void __launch_bounds__(256)
+delta_step_kernel(T* __restrict__ out, const T* __restrict__ proj, int row, int q_off, int g_off,
+                  const float* __restrict__ taps, int ntaps, const float* __restrict__ tails, const float* __restrict__ ab,
+                  const float* __restrict__ a_log, const float* __restrict__ dt_bias, float* __restrict__ state,
+                  const int32_t* __restrict__ slots, const float* __restrict__ gain, float eps, int heads, int kv_heads,
+                  int dim, int vdim, int cols) {
+    __shared__ float qs[256], ks[256], vs[256], part[256], scratch[16];
+    const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int hq = h / (heads / kv_heads), slot = slots[b];
+    const int c = tid % cols, r = tid / cols, slices = 256 / cols;
+    const bool has_col = c < vdim;
+    const int qk = kv_heads * dim, channels = 2 * qk + heads * vdim;
+    float* st = state + (((size_t)slot * heads + h) * dim) * vdim;
+    float S[RPT];
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+        const int rw = r * RPT + i;
+        S[i] = (has_col && rw < dim) ? st[(size_t)rw * vdim + c] : 0.f;
+    }
+    const T* x = proj + (size_t)b * row;
+    const float* tail = tails + (size_t)slot * (ntaps - 1) * channels;
+    for (int e = tid; e < 2 * dim + vdim; e += 256) {
+        const int ch = e < dim ? hq * dim + e : e < 2 * dim ? qk + hq * dim + (e - dim) : 2 * qk + h * vdim + (e - 2 * dim);
+        float y = 0.f;
+        for (int d = ntaps - 1; d >= 1; --d) y += taps[(size_t)ch * ntaps + (ntaps - 1 - d)] * tail[(size_t)(ntaps - 1 - d) * channels + ch];
+        y += taps[(size_t)ch * ntaps + ntaps - 1] * to_f32(x[q_off + ch]);
+        const float a = silu_f(y);
+        if (e < dim) qs[e] = a; else if (e < 2 * dim) ks[e - dim] = a; else vs[e - 2 * dim] = a;
+    }
+    __syncthreads();
+    float sq = 0.f, sk = 0.f;
+    for (int e = tid; e < dim; e += 256) {
+        sq += qs[e] * qs[e];
+        sk += ks[e] * ks[e];
+    }
+    sq = block_sum(sq, scratch);
+    sk = block_sum(sk, scratch);
+    const float fq = rsqrtf((float)dim) / sqrtf(sq + 1e-6f), fk = 1.f / sqrtf(sk + 1e-6f);
+    const float g = expf(-expf(a_log[h]) * softplus_f(ab[(size_t)b * 2 * heads + h] + dt_bias[h]));
+    const float beta = 1.f / (1.f + expf(-ab[(size_t)b * 2 * heads + heads + h]));
+    float kk[RPT], d4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+        const int rw = r * RPT + i;
+        kk[i] = rw < dim ? ks[rw] * fk : 0.f;
+        S[i] *= g;
+        d4[i & 3] += S[i] * kk[i];
+    }
+    part[tid] = (d4[0] + d4[1]) + (d4[2] + d4[3]);
+    __syncthreads();
+    float dot = 0.f;
+    for (int j = 0; j < slices; ++j) dot += part[j * cols + c];
+    const float u = beta * ((has_col ? vs[c] : 0.f) - dot);
+    __syncthreads();                                          // part is written again
+    float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+        const int rw = r * RPT + i;
+        S[i] += kk[i] * u;
+        o4[i & 3] += S[i] * (rw < dim ? qs[rw] * fq : 0.f);
+        if (has_col && rw < dim) st[(size_t)rw * vdim + c] = S[i];
+    }
+    part[tid] = (o4[0] + o4[1]) + (o4[2] + o4[3]);
+    __syncthreads();
+    float o = 0.f;
+    for (int j = 0; j < slices; ++j) o += part[j * cols + c];
+    const float ss = block_sum((r == 0 && has_col) ? o * o : 0.f, scratch);
+    if (r == 0 && has_col) {
+        const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
+        const float gate = to_f32(x[g_off + h * vdim + c]);
+        from_f32(out + (size_t)b * heads * vdim + (size_t)h * vdim + c, o * inv * gain[c] * silu_f(gate));
+    }
+}
+
+static int delta_step_cols(int vdim) {
+    int cols = 32;
+    while (cols < vdim) cols *= 2;
+    return cols;
+}
+
+extern "C" int ri_delta_step_fits(int dim, int vdim) {
+    if (dim < 1 || dim > 256 || vdim < 1 || vdim > 256) return 0;
+    const int slices = 256 / delta_step_cols(vdim);
+    return (dim + slices - 1) / slices <= 64;
+}
+
+extern "C" int ri_delta_step(void* out, const void* proj, int act_dtype, int row, int q_off, int g_off, const float* taps,
+                             int ntaps, float* tails, const float* ab, const float* a_log, const float* dt_bias,
+                             float* state, const int32_t* cu_seqlens, const int32_t* slots, const float* gain, float eps,
+                             int seqs, int heads, int kv_heads, int dim, int vdim, void* stream) {
+    RI_REQUIRE(seqs > 0 && seqs <= 65535 && heads > 0 && heads <= 65535 && kv_heads > 0 && heads % kv_heads == 0,
+               "delta_step: %d sequences, %d heads, %d kv heads", seqs, heads, kv_heads);
+    RI_REQUIRE(ri_delta_step_fits(dim, vdim), "delta_step: heads of %d x %d", dim, vdim);
+    RI_REQUIRE(ntaps >= 1 && ntaps <= DELTA_MAX_TAPS, "delta_step: %d taps, the kernels take 1 to %d", ntaps, DELTA_MAX_TAPS);
+    const long channels = 2L * kv_heads * dim + (long)heads * vdim;
+    RI_REQUIRE(q_off >= 0 && q_off + channels <= row && g_off >= 0 && g_off + (long)heads * vdim <= row,
+               "delta_step: %ld channels at column %d and the gate at %d of rows of %d", channels, q_off, g_off, row);
+    RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "delta_step: dtype %d", act_dtype);
+    hipStream_t s = (hipStream_t)stream;
+    const int cols = delta_step_cols(vdim), slices = 256 / cols, rpt = (dim + slices - 1) / slices;
+    const dim3 grid(heads, seqs);
+#define RI_DSTEP_GO(T, R) delta_step_kernel<T, R><<<grid, 256, 0, s>>>((T*)out, (const T*)proj, row, q_off, g_off, taps, ntaps, \
+                                                                    tails, ab, a_log, dt_bias, state, slots, gain, eps, heads,   \
+                                                                    kv_heads, dim, vdim, cols)
+    if (act_dtype == RI_F32) {
+        if (rpt <= 8) RI_DSTEP_GO(float, 8); else if (rpt <= 16) RI_DSTEP_GO(float, 16); else if (rpt <= 32) RI_DSTEP_GO(float, 32); else RI_DSTEP_GO(float, 64);
+    } else {
+        if (rpt <= 8) RI_DSTEP_GO(bf16_t, 8); else if (rpt <= 16) RI_DSTEP_GO(bf16_t, 16); else if (rpt <= 32) RI_DSTEP_GO(bf16_t, 32); else RI_DSTEP_GO(bf16_t, 64);
+    }
+#undef RI_DSTEP_GO
+    RI_LAUNCH_CHECK("delta_step");
+    if (ntaps > 1) {
+        const dim3 tgrid((unsigned)((channels + 255) / 256), seqs);
+        if (act_dtype == RI_F32)
+            delta_tails_kernel<float><<<tgrid, 256, 0, s>>>(tails, (const float*)proj, row, q_off, ntaps, cu_seqlens, slots, (int)channels);
+        else
+            delta_tails_kernel<bf16_t><<<tgrid, 256, 0, s>>>(tails, (const bf16_t*)proj, row, q_off, ntaps, cu_seqlens, slots, (int)channels);
+        RI_LAUNCH_CHECK("delta_tails");
+    }
+    return 0;
+}
+
 extern "C" int ri_delta_prepare(float* qkv, float* gates, const void* proj, int act_dtype, int row, int q_off,
                                 const float* taps, int ntaps, float* tails, const float* ab, const float* a_log,
                                 const float* dt_bias, const int32_t* tok_seq, const int32_t* cu_seqlens,

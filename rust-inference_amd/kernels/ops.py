@@ -49,6 +49,9 @@ _SIGNATURES = {
     "ri_delta_max_dim": [],
     "ri_delta_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                       c_void_p],
+    "ri_delta_step_fits": [c_int, c_int],
+    "ri_delta_step": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                      c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_experts_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ri_experts_activate": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
     "ri_experts_sort": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -503,6 +506,33 @@ def delta_scan(qkv, gates, state, cu_seqlens, slots, heads: int, kv_heads: int, 
           _dev(gates, "gates", torch.float32, (tokens, 2 * heads)), _dev(state, "state", torch.float32),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
           seqs, tokens, heads, kv_heads, dim, vdim, _stream())
+    return out
+
+
+def delta_step_fits(dim: int, vdim: int) -> bool:
+    """Whether ``delta_step`` takes these head sizes (host code only: it needs no GPU)."""
+    return bool(_get("ri_delta_step_fits")(int(dim), int(vdim)))
+
+
+def delta_step(proj, q_off: int, g_off: int, taps, tails, ab, a_log, dt_bias, state, cu_seqlens, slots, gain, eps: float,
+               heads: int, kv_heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """One new token a sequence (row ``b`` of ``proj`` and ``ab`` belongs to ``slots[b]``): what ``delta_prepare`` and
+    ``delta_scan`` compute, the per-head RMS norm and the gate ``silu(g)`` (at column ``g_off`` of ``proj``) in one
+    kernel, and the tails moved on; ``[seqs, heads * vdim]`` in the dtype of ``proj``."""
+    seqs, row = proj.shape
+    channels = 2 * kv_heads * dim + heads * vdim
+    ntaps = taps.shape[1]
+    if state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, vdim):
+        raise ShapeError(f"the state is {list(state.shape)}, not [slots, {heads}, {dim}, {vdim}]")
+    if tails.dim() != 3 or tuple(tails.shape[1:]) != (ntaps - 1, channels):
+        raise ShapeError(f"the convolutions' tails are {list(tails.shape)}, not [slots, {ntaps - 1}, {channels}]")
+    out = torch.empty((seqs, heads * vdim), dtype=proj.dtype, device=proj.device)
+    _call("ri_delta_step", _dev(out, "out"), _dev(proj, "proj"), code(proj.dtype), row, q_off, g_off,
+          _dev(taps, "taps", torch.float32, (channels, ntaps)), ntaps, _dev(tails, "tails", torch.float32),
+          _dev(ab, "ab", torch.float32, (seqs, 2 * heads)), _dev(a_log, "a_log", torch.float32, (heads,)),
+          _dev(dt_bias, "dt_bias", torch.float32, (heads,)), _dev(state, "state", torch.float32),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
+          _dev(gain, "gain", torch.float32, (vdim,)), float(eps), seqs, heads, kv_heads, dim, vdim, _stream())
     return out
 
 

@@ -397,3 +397,43 @@ def test_an_experts_rows_activated_without_weights(ops):
     g, u = np.minimum(gu[:, 0], 1.1), np.clip(gu[:, 1], -1.1, 1.1)
     got = ops.experts_activate(t(gu.reshape(7, -1)), None, 20, 1.1)
     close(got, g * P.sigmoid(1.702 * g) * (u + 1.0), F32)
+
+
+# ---------------------------------------------------------------- the delta rule's one-token kernel
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H, G, dk, dv, K", [(4, 2, 12, 20, 4), (2, 1, 64, 48, 3), (3, 3, 5, 70, 2), (2, 2, 128, 128, 4),
+                                             (1, 1, 60, 130, 1), (2, 1, 256, 40, 5), (1, 1, 9, 256, 2)])
+def test_delta_step_of_one_token_a_sequence(ops, dtype, H, G, dk, dv, K):
+    """Against the plain functions, and against the kernels of the prompt path on the same inputs: states that are not
+    zero, on slots in another order, tails partly filled."""
+    assert ops.delta_step_fits(dk, dv)
+    rng = np.random.default_rng(H * 13 + dv)
+    B = 3
+    c = delta_case(rng, B, H, G, dk, dv, K)
+    if dtype == torch.bfloat16:
+        c["proj"] = bf16_round(c["proj"])
+    slots = [3, 0, 4]
+    tails, state, gain = rng.normal(size=(5, K - 1, c["C"])), rng.normal(size=(5, H, dk, dv)) * 0.3, 1 + 0.1 * rng.normal(size=dv)
+    plain_tails = [tails[s].copy() for s in slots]
+    qkv, gates = plain_prepare(c, H, G, dk, dv, K, [1] * B, plain_tails)
+    want_state, want = state.copy(), np.zeros((B, H, dv))
+    for b in range(B):
+        for h in range(H):
+            hq = h // (H // G)
+            o = P.delta_recurrence(qkv[b:b + 1, hq * dk:(hq + 1) * dk], qkv[b:b + 1, (G + hq) * dk:(G + hq + 1) * dk],
+                                   qkv[b:b + 1, 2 * G * dk + h * dv:2 * G * dk + (h + 1) * dv], gates[b:b + 1, H + h],
+                                   gates[b:b + 1, h], want_state[slots[b], h])
+            want[b, h] = P.rms_norm(o[0], gain, 1e-5) * P.silu(c["proj"][b, c["C"] + h * dv:c["C"] + (h + 1) * dv])
+    dev_tails, dev_state = t(tails), t(state)
+    got = ops.delta_step(t(c["proj"], dtype), 0, c["C"], t(c["taps"]), dev_tails, t(c["ab"]), t(c["a_log"]), t(c["dt_bias"]),
+                         dev_state, t(np.arange(B + 1), torch.int32), t(slots, torch.int32), t(gain), 1e-5, H, G, dk, dv)
+    close(got, want.reshape(B, -1), 2e-5 if dtype == torch.float32 else BF16_OUT, "outputs")
+    close(dev_state, want_state, 1e-5, "state")
+    for s, w in zip(slots, plain_tails):
+        if K > 1:
+            close(dev_tails[s], w, 1e-7, "tail")
+
+
+def test_delta_step_does_not_fit_every_size(ops):
+    assert not ops.delta_step_fits(300, 64) and not ops.delta_step_fits(64, 300) and not ops.delta_step_fits(100, 130)
+    assert ops.delta_step_fits(256, 64) and ops.delta_step_fits(64, 256)
