@@ -270,8 +270,22 @@ delta_step_kernel(T* __restrict__ out, const T* __restrict__ proj, int row, int 
     for (int e = tid; e < 2 * dim + vdim; e += 256) {
         const int ch = e < dim ? hq * dim + e : e < 2 * dim ? qk + hq * dim + (e - dim) : 2 * qk + h * vdim + (e - 2 * dim);
         float y = 0.f;
-        for (int d = ntaps - 1; d >= 1; --d) y += taps[(size_t)ch * ntaps + (ntaps - 1 - d)] * tail[(size_t)(ntaps - 1 - d) * channels + ch];
-        y += taps[(size_t)ch * ntaps + ntaps - 1] * to_f32(x[q_off + ch]);
+        if (ntaps <= 4) {                                     // the usual few taps: every load asked for before any is used
+            const float* tail_safe = ntaps > 1 ? tail : taps;
+            float xv[3], wv[3];
+#pragma unroll
+            for (int d = 1; d <= 3; ++d) {
+                xv[d - 1] = tail_safe[(size_t)max(ntaps - 1 - d, 0) * channels + ch];
+                wv[d - 1] = taps[(size_t)ch * ntaps + max(ntaps - 1 - d, 0)];
+            }
+            const float w0 = taps[(size_t)ch * ntaps + ntaps - 1], x0 = to_f32(x[q_off + ch]);
+#pragma unroll
+            for (int d = 3; d >= 1; --d) y += d < ntaps ? wv[d - 1] * xv[d - 1] : 0.f;
+            y += w0 * x0;
+        } else {
+            for (int d = ntaps - 1; d >= 1; --d) y += taps[(size_t)ch * ntaps + (ntaps - 1 - d)] * tail[(size_t)(ntaps - 1 - d) * channels + ch];
+            y += taps[(size_t)ch * ntaps + ntaps - 1] * to_f32(x[q_off + ch]);
+        }
         const float a = silu_f(y);
         if (e < dim) qs[e] = a; else if (e < 2 * dim) ks[e - dim] = a; else vs[e - 2 * dim] = a;
     }
