@@ -154,8 +154,10 @@ delta_scan_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
     float S[RPT];
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
+        // (no load in a branch: the address is pulled back inside the state and the value dropped afterwards)
         const int rw = r * RPT + i;
-        S[i] = (has_col && rw < dim) ? st[(size_t)rw * vdim + col] : 0.f;
+        const float v = st[(size_t)min(rw, dim - 1) * vdim + min(col, vdim - 1)];
+        S[i] = (has_col && rw < dim) ? v : 0.f;
     }
 
     float fq[QR], fk[QR], fv[VR], fg = 0.f;
@@ -240,33 +242,44 @@ delta_scan_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
 }
 
 // One new token a sequence: the convolutions, the unit norms, the gates, the step on the state, the per-head norm
-// and the output gate in one kernel.  A workgroup owns one (sequence, head): `cols` columns (vdim rounded up to a power
-// of two, 32 at least) x 256 / cols slices of rows, a thread RPT rows of one column in registers; consecutive lanes hold
-// consecutive columns, so the state streams in and out in whole lines.  The sums over rows meet through LDS, slice after
-// slice.  The convolutions' tails are read here and moved on by delta_tails_kernel afterwards (the heads that share a
-// q/k head all read its tail).
+// and the output gate in one kernel.  A workgroup owns one (sequence, head): `groups` threads across a row of the
+// state, four columns each (16-byte loads and stores of whole lines), x 256 / groups slices of rows, a thread RPT rows
+// in registers.  The sums over rows meet through LDS, slice after slice.  The convolutions' tails are read here and
+// moved on by delta_tails_kernel afterwards (the heads that share a q/k head all read its tail).
 template <typename T, int RPT>
 __global__ void __launch_bounds__(256)
 delta_step_kernel(T* __restrict__ out, const T* __restrict__ proj, int row, int q_off, int g_off,
                   const float* __restrict__ taps, int ntaps, const float* __restrict__ tails, const float* __restrict__ ab,
                   const float* __restrict__ a_log, const float* __restrict__ dt_bias, float* __restrict__ state,
                   const int32_t* __restrict__ slots, const float* __restrict__ gain, float eps, int heads, int kv_heads,
-                  int dim, int vdim, int cols) {
-    __shared__ float qs[256], ks[256], vs[256], part[256], scratch[16];
+                  int dim, int vdim, int groups) {
+    __shared__ float qs[256], ks[256], vs[256], scratch[16];
+    __shared__ float4 part[256];
     const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
     const int hq = h / (heads / kv_heads), slot = slots[b];
-    const int c = tid % cols, r = tid / cols, slices = 256 / cols;
-    const bool has_col = c < vdim;
+    const int grp = tid % groups, r = tid / groups, slices = 256 / groups, c0 = grp * 4;
+    const bool has_col = c0 < vdim;                           // vdim is a multiple of 4: all four columns or none
     const int qk = kv_heads * dim, channels = 2 * qk + heads * vdim;
     float* st = state + (((size_t)slot * heads + h) * dim) * vdim;
-    float S[RPT];
+    float4 S[RPT];
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
+        // (no load in a branch: the address is pulled back inside the state and the value dropped afterwards)
         const int rw = r * RPT + i;
-        S[i] = (has_col && rw < dim) ? st[(size_t)rw * vdim + c] : 0.f;
+        const float4 v = *reinterpret_cast<const float4*>(st + (size_t)min(rw, dim - 1) * vdim + min(c0, vdim - 4));
+        S[i] = (has_col && rw < dim) ? v : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     const T* x = proj + (size_t)b * row;
     const float* tail = tails + (size_t)slot * (ntaps - 1) * channels;
+    // everything the end of the kernel reads from memory is asked for here, so that no load is waited for on its own
+    const float a_in = ab[(size_t)b * 2 * heads + h], b_in = ab[(size_t)b * 2 * heads + heads + h];
+    const float a_exp = a_log[h], a_bias = dt_bias[h];
+    float gate[4], gain_c[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        gate[j] = to_f32(x[g_off + h * vdim + min(c0, vdim - 4) + j]);
+        gain_c[j] = gain[min(c0, vdim - 4) + j];
+    }
     for (int e = tid; e < 2 * dim + vdim; e += 256) {
         const int ch = e < dim ? hq * dim + e : e < 2 * dim ? qk + hq * dim + (e - dim) : 2 * qk + h * vdim + (e - 2 * dim);
         float y = 0.f;
@@ -298,39 +311,52 @@ delta_step_kernel(T* __restrict__ out, const T* __restrict__ proj, int row, int 
     sq = block_sum(sq, scratch);
     sk = block_sum(sk, scratch);
     const float fq = rsqrtf((float)dim) / sqrtf(sq + 1e-6f), fk = 1.f / sqrtf(sk + 1e-6f);
-    const float g = expf(-expf(a_log[h]) * softplus_f(ab[(size_t)b * 2 * heads + h] + dt_bias[h]));
-    const float beta = 1.f / (1.f + expf(-ab[(size_t)b * 2 * heads + heads + h]));
-    float kk[RPT], d4[4] = {0.f, 0.f, 0.f, 0.f};
+    const float g = expf(-expf(a_exp) * softplus_f(a_in + a_bias));
+    const float beta = 1.f / (1.f + expf(-b_in));
+    float kk[RPT];
+    float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
         const int rw = r * RPT + i;
         kk[i] = rw < dim ? ks[rw] * fk : 0.f;
-        S[i] *= g;
-        d4[i & 3] += S[i] * kk[i];
+        S[i].x *= g; S[i].y *= g; S[i].z *= g; S[i].w *= g;
+        d.x += S[i].x * kk[i]; d.y += S[i].y * kk[i]; d.z += S[i].z * kk[i]; d.w += S[i].w * kk[i];
     }
-    part[tid] = (d4[0] + d4[1]) + (d4[2] + d4[3]);
+    part[tid] = d;
     __syncthreads();
-    float dot = 0.f;
-    for (int j = 0; j < slices; ++j) dot += part[j * cols + c];
-    const float u = beta * ((has_col ? vs[c] : 0.f) - dot);
+    float4 dot = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int j = 0; j < slices; ++j) {                        // slice after slice: the same order for every column
+        const float4 p = part[j * groups + grp];
+        dot.x += p.x; dot.y += p.y; dot.z += p.z; dot.w += p.w;
+    }
+    const int cv = min(c0, vdim - 4);
+    const float4 u = make_float4(beta * (vs[cv] - dot.x), beta * (vs[cv + 1] - dot.y), beta * (vs[cv + 2] - dot.z),
+                                 beta * (vs[cv + 3] - dot.w));
     __syncthreads();                                          // part is written again
-    float o4[4] = {0.f, 0.f, 0.f, 0.f};
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
         const int rw = r * RPT + i;
-        S[i] += kk[i] * u;
-        o4[i & 3] += S[i] * (rw < dim ? qs[rw] * fq : 0.f);
-        if (has_col && rw < dim) st[(size_t)rw * vdim + c] = S[i];
+        const float qq = rw < dim ? qs[rw] * fq : 0.f;
+        S[i].x += kk[i] * u.x; S[i].y += kk[i] * u.y; S[i].z += kk[i] * u.z; S[i].w += kk[i] * u.w;
+        o.x += S[i].x * qq; o.y += S[i].y * qq; o.z += S[i].z * qq; o.w += S[i].w * qq;
+        if (has_col && rw < dim) *reinterpret_cast<float4*>(st + (size_t)rw * vdim + c0) = S[i];
     }
-    part[tid] = (o4[0] + o4[1]) + (o4[2] + o4[3]);
+    part[tid] = o;
     __syncthreads();
-    float o = 0.f;
-    for (int j = 0; j < slices; ++j) o += part[j * cols + c];
-    const float ss = block_sum((r == 0 && has_col) ? o * o : 0.f, scratch);
+    o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int j = 0; j < slices; ++j) {
+        const float4 p = part[j * groups + grp];
+        o.x += p.x; o.y += p.y; o.z += p.z; o.w += p.w;
+    }
+    const float ss = block_sum((r == 0 && has_col) ? (o.x * o.x + o.y * o.y) + (o.z * o.z + o.w * o.w) : 0.f, scratch);
     if (r == 0 && has_col) {
         const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
-        const float gate = to_f32(x[g_off + h * vdim + c]);
-        from_f32(out + (size_t)b * heads * vdim + (size_t)h * vdim + c, o * inv * gain[c] * silu_f(gate));
+        T* to = out + (size_t)b * heads * vdim + (size_t)h * vdim + c0;
+        from_f32(to, o.x * inv * gain_c[0] * silu_f(gate[0]));
+        from_f32(to + 1, o.y * inv * gain_c[1] * silu_f(gate[1]));
+        from_f32(to + 2, o.z * inv * gain_c[2] * silu_f(gate[2]));
+        from_f32(to + 3, o.w * inv * gain_c[3] * silu_f(gate[3]));
     }
 }
 
@@ -341,9 +367,9 @@ static int delta_step_cols(int vdim) {
 }
 
 extern "C" int ri_delta_step_fits(int dim, int vdim) {
-    if (dim < 1 || dim > 256 || vdim < 1 || vdim > 256) return 0;
-    const int slices = 256 / delta_step_cols(vdim);
-    return (dim + slices - 1) / slices <= 64;
+    if (dim < 1 || dim > 256 || vdim < 4 || vdim > 256 || vdim % 4) return 0;
+    const int slices = 256 / (delta_step_cols(vdim) / 4);
+    return (dim + slices - 1) / slices <= 16;
 }
 
 extern "C" int ri_delta_step(void* out, const void* proj, int act_dtype, int row, int q_off, int g_off, const float* taps,
@@ -359,15 +385,15 @@ extern "C" int ri_delta_step(void* out, const void* proj, int act_dtype, int row
                "delta_step: %ld channels at column %d and the gate at %d of rows of %d", channels, q_off, g_off, row);
     RI_REQUIRE(act_dtype == RI_F32 || act_dtype == RI_BF16, "delta_step: dtype %d", act_dtype);
     hipStream_t s = (hipStream_t)stream;
-    const int cols = delta_step_cols(vdim), slices = 256 / cols, rpt = (dim + slices - 1) / slices;
+    const int groups = delta_step_cols(vdim) / 4, slices = 256 / groups, rpt = (dim + slices - 1) / slices;
     const dim3 grid(heads, seqs);
 #define RI_DSTEP_GO(T, R) delta_step_kernel<T, R><<<grid, 256, 0, s>>>((T*)out, (const T*)proj, row, q_off, g_off, taps, ntaps, \
                                                                     tails, ab, a_log, dt_bias, state, slots, gain, eps, heads,   \
-                                                                    kv_heads, dim, vdim, cols)
+                                                                    kv_heads, dim, vdim, groups)
     if (act_dtype == RI_F32) {
-        if (rpt <= 8) RI_DSTEP_GO(float, 8); else if (rpt <= 16) RI_DSTEP_GO(float, 16); else if (rpt <= 32) RI_DSTEP_GO(float, 32); else RI_DSTEP_GO(float, 64);
+        if (rpt <= 4) RI_DSTEP_GO(float, 4); else if (rpt <= 8) RI_DSTEP_GO(float, 8); else RI_DSTEP_GO(float, 16);
     } else {
-        if (rpt <= 8) RI_DSTEP_GO(bf16_t, 8); else if (rpt <= 16) RI_DSTEP_GO(bf16_t, 16); else if (rpt <= 32) RI_DSTEP_GO(bf16_t, 32); else RI_DSTEP_GO(bf16_t, 64);
+        if (rpt <= 4) RI_DSTEP_GO(bf16_t, 4); else if (rpt <= 8) RI_DSTEP_GO(bf16_t, 8); else RI_DSTEP_GO(bf16_t, 16);
     }
 #undef RI_DSTEP_GO
     RI_LAUNCH_CHECK("delta_step");
