@@ -60,7 +60,7 @@ P_B = {"architecture": "Pisulorn", "vocab": 300, "width": 64, "norm": {"eps": 1e
 # times, a window of exactly one page, one expert chosen of many, convolutions of one tap (no tail at all).
 P_C = {"architecture": "Pisulorn", "vocab": 157, "width": 128, "norm": {"eps": 1e-5}, "streams": 1,
        "loop": {"start": 0, "stop": 1, "times": 3},
-       "layers": [attention(8, 2, 64, 64, 0.11, 32, {"coef": 0.3, "every": 64}, moe(9, 1, 56, 1.2)),
+       "layers": [attention(8, 4, 64, 64, 0.11, 32, {"coef": 0.25, "every": 48}, moe(9, 1, 56, 1.2)),
                   delta(2, 1, 64, 48, 1, dense(96)),
                   delta(3, 3, 20, 72, 5, dense(40))]}
 CONFIGS = {"A": P_A, "B": P_B, "C": P_C}
