@@ -127,8 +127,10 @@ int ri_delta_prepare(float* qkv, float* gates, const void* proj, int act_dtype, 
 // Per sequence and head, over the sequence's new tokens in order: S <- g S; u = beta (v - S^T k); S <- S + k u^T;
 // o = S^T q.  state: float32 [slots, heads, dim, vdim]; out: float32 [tokens, heads * vdim].
 int ri_delta_max_dim();
+// slices: over how many lanes a column's rows are spread, 4 or 8; 0: by the size of the launch.
 int ri_delta_scan(float* out, const float* qkv, const float* gates, float* state, const int32_t* cu_seqlens,
-                  const int32_t* slots, int seqs, int tokens, int heads, int kv_heads, int dim, int vdim, void* stream);
+                  const int32_t* slots, int seqs, int tokens, int heads, int kv_heads, int dim, int vdim, int slices,
+                  void* stream);
 
 // One new token a sequence (token b is sequence b's; cu_seqlens is 0, 1, .., seqs): ri_delta_prepare, ri_delta_scan, the
 // per-head RMS norm over vdim with `gain` and the gate silu(g) (read from proj rows at column g_off) in one kernel, then

@@ -119,32 +119,44 @@ __device__ __forceinline__ float quad_sum(float v) {
     return v;
 }
 
-// The walk.  A workgroup owns one (sequence, value head) and 64 columns of its state: 64 columns x 4 slices of
-// rows; a thread keeps RPT rows of one column in registers (rows r * RPT ..+RPT of slice r; rows past dim are
-// zeros that stay zeros).  Tokens come through LDS in blocks of DELTA_BLOCK, the next block's loads in flight
-// while a block is walked.  The two sums over rows of a token meet over the four lanes of a column.
-template <int RPT>
+// The same over the SL = 4 or 8 lanes of a column: after the quads, the mirror image inside every eight lanes
+// (lane i takes lane 7 - i: the other quad, all of whose lanes hold its sum).
+template <int SL>
+__device__ __forceinline__ float slices_sum(float v) {
+    v = quad_sum(v);
+    if (SL == 8) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));
+    return v;
+}
+
+// The walk.  A workgroup owns one (sequence, value head) and 256 / SL columns of its state: that many columns x SL
+// slices of rows (4 or 8); a thread keeps RPT rows of one column in registers (rows r * RPT ..+RPT of slice r; rows
+// past dim are zeros that stay zeros).  Tokens come through LDS in blocks of DELTA_BLOCK, the next block's loads in
+// flight while a block is walked.  The two sums over rows of a token meet over the SL lanes of a column.  A token costs
+// a wavefront 4 RPT vector instructions and nothing hides them, so eight slices halve a token's time; they also
+// double the workgroups that each stage q and k, which is what counts once the machine is full: the launch chooses.
+template <int RPT, int SL>
 struct DeltaLds {
-    static constexpr int DELTA_BLOCK = RPT >= 64 ? 8 : 16;    // tokens a block: two buffers stay inside 64 KB
-    static constexpr int QS = RPT + 4;                        // stride of a slice of q or k: no bank conflicts between the four slices
-    float q[DELTA_BLOCK][4][QS];
-    float k[DELTA_BLOCK][4][QS];
-    float v[DELTA_BLOCK][64];
+    static constexpr int DELTA_BLOCK = RPT * SL >= 256 ? 8 : 16;    // tokens a block: two buffers stay inside 64 KB
+    static constexpr int QS = RPT + 4;                        // stride of a slice of q or k: no bank conflicts between the slices
+    static constexpr int COLS = 256 / SL;
+    float q[DELTA_BLOCK][SL][QS];
+    float k[DELTA_BLOCK][SL][QS];
+    float v[DELTA_BLOCK][COLS];
     float g[DELTA_BLOCK], beta[DELTA_BLOCK];
 };
 
-template <int RPT>
+template <int RPT, int SL>
 __global__ void __launch_bounds__(256)
 delta_scan_kernel(float* __restrict__ out, const float* __restrict__ qkv, const float* __restrict__ gates,
                   float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
                   int heads, int kv_heads, int dim, int vdim) {
-    __shared__ DeltaLds<RPT> lds[2];
-    constexpr int DELTA_BLOCK = DeltaLds<RPT>::DELTA_BLOCK;
-    constexpr int QR = DELTA_BLOCK * 4 * RPT / 256;           // elements of q (and of k) a thread fetches per block
-    constexpr int VR = DELTA_BLOCK * 64 / 256;
-    const int b = blockIdx.x / heads, h = blockIdx.x % heads, col0 = blockIdx.y * 64;
+    __shared__ DeltaLds<RPT, SL> lds[2];
+    constexpr int DELTA_BLOCK = DeltaLds<RPT, SL>::DELTA_BLOCK, COLS = DeltaLds<RPT, SL>::COLS;
+    constexpr int QR = DELTA_BLOCK * SL * RPT / 256;          // elements of q (and of k) a thread fetches per block
+    constexpr int VR = DELTA_BLOCK * COLS / 256;
+    const int b = blockIdx.x / heads, h = blockIdx.x % heads, col0 = blockIdx.y * COLS;
     const int hq = h / (heads / kv_heads);
-    const int tid = threadIdx.x, r = tid & 3, col = col0 + (tid >> 2);
+    const int tid = threadIdx.x, r = tid & (SL - 1), col = col0 + tid / SL;
     const bool has_col = col < vdim;
     const int t0 = cu_seqlens[b], n = cu_seqlens[b + 1] - t0;
     if (n <= 0) return;
@@ -164,7 +176,7 @@ delta_scan_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
     auto fetch = [&](int first) {                             // the block of tokens first ..+DELTA_BLOCK, into registers
 #pragma unroll
         for (int e = 0; e < QR; ++e) {
-            const int at = e * 256 + tid, tk = at / (4 * RPT), rw = at % (4 * RPT);
+            const int at = e * 256 + tid, tk = at / (SL * RPT), rw = at % (SL * RPT);
             const bool ok = first + tk < n && rw < dim;
             const float* p = qkv + (size_t)(t0 + min(first + tk, n - 1)) * channels + (size_t)hq * dim + min(rw, dim - 1);
             const float a = p[0], c = p[qk];
@@ -173,7 +185,7 @@ delta_scan_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
         }
 #pragma unroll
         for (int e = 0; e < VR; ++e) {
-            const int at = e * 256 + tid, tk = at >> 6, cc = col0 + (at & 63);
+            const int at = e * 256 + tid, tk = at / COLS, cc = col0 + at % COLS;
             const float a = qkv[(size_t)(t0 + min(first + tk, n - 1)) * channels + 2 * qk + (size_t)h * vdim + min(cc, vdim - 1)];
             fv[e] = a;
         }
@@ -182,17 +194,17 @@ delta_scan_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
             fg = gates[(size_t)(t0 + min(first + tk, n - 1)) * 2 * heads + (tid & 1) * heads + h];
         }
     };
-    auto stage = [&](DeltaLds<RPT>& l) {
+    auto stage = [&](DeltaLds<RPT, SL>& l) {
 #pragma unroll
         for (int e = 0; e < QR; ++e) {
-            const int at = e * 256 + tid, tk = at / (4 * RPT), rw = at % (4 * RPT);
+            const int at = e * 256 + tid, tk = at / (SL * RPT), rw = at % (SL * RPT);
             l.q[tk][rw / RPT][rw % RPT] = fq[e];
             l.k[tk][rw / RPT][rw % RPT] = fk[e];
         }
 #pragma unroll
         for (int e = 0; e < VR; ++e) {
             const int at = e * 256 + tid;
-            l.v[at >> 6][at & 63] = fv[e];
+            l.v[at / COLS][at % COLS] = fv[e];
         }
         if (tid < 2 * DELTA_BLOCK) {
             if (tid & 1) l.beta[tid >> 1] = fg; else l.g[tid >> 1] = fg;
@@ -206,7 +218,7 @@ delta_scan_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
     for (int first = 0; first < n; first += DELTA_BLOCK) {
         const bool more = first + DELTA_BLOCK < n;
         fetch(more ? first + DELTA_BLOCK : first);            // (always issued: no load in a branch)
-        const DeltaLds<RPT>& l = lds[cur];
+        const DeltaLds<RPT, SL>& l = lds[cur];
         const int count = min(DELTA_BLOCK, n - first);
 #pragma unroll 2
         for (int tk = 0; tk < count; ++tk) {
@@ -219,15 +231,15 @@ delta_scan_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
                 S[i] *= g;
                 d4[i & 3] += S[i] * kk[i];
             }
-            const float dot = quad_sum((d4[0] + d4[1]) + (d4[2] + d4[3]));
-            const float u = beta * (l.v[tk][tid >> 2] - dot);
+            const float dot = slices_sum<SL>((d4[0] + d4[1]) + (d4[2] + d4[3]));
+            const float u = beta * (l.v[tk][tid / SL] - dot);
             float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
                 S[i] += kk[i] * u;
                 o4[i & 3] += S[i] * l.q[tk][r][i];
             }
-            const float o = quad_sum((o4[0] + o4[1]) + (o4[2] + o4[3]));
+            const float o = slices_sum<SL>((o4[0] + o4[1]) + (o4[2] + o4[3]));
             if (r == 0 && has_col) out[(size_t)(t0 + first + tk) * heads * vdim + (size_t)h * vdim + col] = o;
         }
         stage(lds[cur ^ 1]);
@@ -452,20 +464,32 @@ extern "C" int ri_delta_max_dim() { return 256; }
 
 extern "C" int ri_delta_scan(float* out, const float* qkv, const float* gates, float* state, const int32_t* cu_seqlens,
                              const int32_t* slots, int seqs, int tokens, int heads, int kv_heads, int dim, int vdim,
-                             void* stream) {
+                             int slices, void* stream) {
+    RI_REQUIRE(slices == 0 || slices == 4 || slices == 8, "delta_scan: %d slices of rows (4, 8, or 0 for the launch's choice)", slices);
     RI_REQUIRE(tokens > 0 && seqs > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && vdim > 0,
                "delta_scan: tokens %d, sequences %d, heads %d, kv heads %d", tokens, seqs, heads, kv_heads);
     RI_REQUIRE(dim >= 1 && dim <= 256, "delta_scan: key heads of %d, the kernel takes 1 to 256", dim);
-    RI_REQUIRE((long)seqs * heads <= 2147483647L && (vdim + 63) / 64 <= 65535, "delta_scan: the grid");
+    RI_REQUIRE((long)seqs * heads <= 2147483647L && (vdim + 31) / 32 <= 65535, "delta_scan: the grid");
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid((unsigned)(seqs * heads), (unsigned)((vdim + 63) / 64));
-    const int need = (dim + 3) / 4;
-#define RI_DELTA_GO(R) delta_scan_kernel<R><<<grid, 256, 0, s>>>(out, qkv, gates, state, cu_seqlens, slots, heads, kv_heads, dim, vdim)
-    if (need <= 4) RI_DELTA_GO(4);
-    else if (need <= 8) RI_DELTA_GO(8);
-    else if (need <= 16) RI_DELTA_GO(16);
-    else if (need <= 32) RI_DELTA_GO(32);
-    else RI_DELTA_GO(64);
+    // eight slices of rows while the workgroups of four would leave compute units idle (a token's time halves), four
+    // once they fill the machine (half the workgroups stage q and k)
+    const bool eight = slices ? slices == 8 : (long)seqs * heads * ((vdim + 63) / 64) <= (long)ri_compute_units() && dim >= 8;
+    const int sl = eight ? 8 : 4, cols = 256 / sl;
+    const dim3 grid((unsigned)(seqs * heads), (unsigned)((vdim + cols - 1) / cols));
+    const int need = (dim + sl - 1) / sl;
+#define RI_DELTA_GO(R, SL) delta_scan_kernel<R, SL><<<grid, 256, 0, s>>>(out, qkv, gates, state, cu_seqlens, slots, heads, kv_heads, dim, vdim)
+    if (eight) {
+        if (need <= 4) RI_DELTA_GO(4, 8);
+        else if (need <= 8) RI_DELTA_GO(8, 8);
+        else if (need <= 16) RI_DELTA_GO(16, 8);
+        else RI_DELTA_GO(32, 8);
+    } else {
+        if (need <= 4) RI_DELTA_GO(4, 4);
+        else if (need <= 8) RI_DELTA_GO(8, 4);
+        else if (need <= 16) RI_DELTA_GO(16, 4);
+        else if (need <= 32) RI_DELTA_GO(32, 4);
+        else RI_DELTA_GO(64, 4);
+    }
 #undef RI_DELTA_GO
     RI_LAUNCH_CHECK("delta_scan");
     return 0;

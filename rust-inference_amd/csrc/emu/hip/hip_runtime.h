@@ -158,12 +158,13 @@ static inline int emu_readfirstlane(int v) {
     const uint64_t live = emu::wave_gather(&v, sizeof(int), all);
     return all[__builtin_ctzll(live)];
 }
-// v_mov_b32 with a DPP quad permutation (control 0x00 .. 0xFF: lane q of every four takes the value of lane
-// (control >> 2q) & 3 of the same four); all rows and banks enabled.
+// v_mov_b32 with a DPP control; all rows and banks enabled.  0x00 .. 0xFF: a quad permutation (lane q of every four
+// takes the value of lane (control >> 2q) & 3 of the same four); 0x141: the mirror image inside every eight lanes.
 static inline int emu_mov_dpp_quad(int v, int control) {
     int all[64];
     emu::wave_gather(&v, sizeof(int), all);
     const int lane = emu::self->lane;
+    if (control == 0x141) return all[(lane & ~7) | (7 - (lane & 7))];
     return all[(lane & ~3) | ((control >> (2 * (lane & 3))) & 3)];
 }
 #define __builtin_amdgcn_mov_dpp(v, control, row_mask, bank_mask, bound_ctrl) emu_mov_dpp_quad((v), (control))

@@ -48,7 +48,7 @@ _SIGNATURES = {
                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_delta_max_dim": [],
     "ri_delta_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                      c_void_p],
+                      c_int, c_void_p],
     "ri_delta_step_fits": [c_int, c_int],
     "ri_delta_step": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -492,10 +492,12 @@ def delta_prepare(proj, q_off: int, taps, tails, ab, a_log, dt_bias, tok_seq, cu
     return qkv, gates
 
 
-def delta_scan(qkv, gates, state, cu_seqlens, slots, heads: int, kv_heads: int, dim: int, vdim: int) -> torch.Tensor:
+def delta_scan(qkv, gates, state, cu_seqlens, slots, heads: int, kv_heads: int, dim: int, vdim: int,
+               slices: int = 0) -> torch.Tensor:
     """The gated delta rule over every sequence's new tokens, ``S <- g S; u = beta (v - S^T k); S <- S + k u^T;
     o = S^T q``; float32 ``[T, heads * vdim]``.  ``state: [slots, heads, dim, vdim]`` float32 is read and written at
-    the sequences' slots."""
+    the sequences' slots.  ``slices``: the lanes a column's rows are spread over, 4 or 8 (0: chosen by the size of the
+    launch, which depends on the sequences and heads and not on their tokens)."""
     tokens = qkv.shape[0]
     seqs = slots.shape[0]
     channels = 2 * kv_heads * dim + heads * vdim
@@ -505,7 +507,7 @@ def delta_scan(qkv, gates, state, cu_seqlens, slots, heads: int, kv_heads: int, 
     _call("ri_delta_scan", _dev(out, "out"), _dev(qkv, "qkv", torch.float32, (tokens, channels)),
           _dev(gates, "gates", torch.float32, (tokens, 2 * heads)), _dev(state, "state", torch.float32),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(slots, "slots", torch.int32, (seqs,)),
-          seqs, tokens, heads, kv_heads, dim, vdim, _stream())
+          seqs, tokens, heads, kv_heads, dim, vdim, int(slices), _stream())
     return out
 
 

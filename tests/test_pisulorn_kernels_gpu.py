@@ -177,7 +177,8 @@ def test_delta_prepare_and_the_convolutions_tails(ops, dtype, H, G, dk, dv, K, l
 @pytest.mark.parametrize("H, G, dk, dv, lens", [(4, 2, 12, 20, (1, 7, 3)), (2, 1, 64, 48, (45,)), (3, 3, 5, 70, (2, 18)),
                                                 (1, 1, 100, 130, (20,)), (2, 2, 33, 8, (17, 1)), (1, 1, 130, 16, (9,)),
                                                 (1, 1, 256, 8, (11,))])
-def test_delta_scan(ops, H, G, dk, dv, lens):
+@pytest.mark.parametrize("slices", [0, 4, 8])
+def test_delta_scan(ops, H, G, dk, dv, lens, slices):
     rng = np.random.default_rng(H * 11 + dk)
     T = sum(lens)
     C = 2 * G * dk + H * dv
@@ -198,12 +199,14 @@ def test_delta_scan(ops, H, G, dk, dv, lens):
     assert qkv.shape[1] == C
     cu = np.concatenate([[0], np.cumsum(lens)])
     dev_state = t(state)
-    got = ops.delta_scan(t(qkv), t(np.concatenate([g, beta], 1)), dev_state, t(cu, torch.int32), t(slots, torch.int32), H, G, dk, dv)
+    got = ops.delta_scan(t(qkv), t(np.concatenate([g, beta], 1)), dev_state, t(cu, torch.int32), t(slots, torch.int32), H, G, dk, dv,
+                         slices)
     close(got, want.reshape(T, -1), 1e-5, "outputs")
     close(dev_state, want_state, 1e-5, "state")
 
 
-def test_delta_scan_token_by_token_is_the_walk_in_blocks(ops):
+@pytest.mark.parametrize("slices", [4, 8])
+def test_delta_scan_token_by_token_is_the_walk_in_blocks(ops, slices):
     """The same 37 tokens in one step, and one at a time from the state the step before left: the same bits."""
     rng = np.random.default_rng(5)
     H, G, dk, dv, T = 2, 1, 24, 40, 37
@@ -211,9 +214,9 @@ def test_delta_scan_token_by_token_is_the_walk_in_blocks(ops):
     qkv = np.concatenate([q.reshape(T, -1), k.reshape(T, -1), rng.normal(size=(T, H * dv))], 1)
     gates = np.concatenate([rng.uniform(0.3, 1.0, size=(T, H)), rng.uniform(0.1, 1.0, size=(T, H))], 1)
     one, slot = t(np.zeros((2, H, dk, dv))), t([1], torch.int32)
-    whole = ops.delta_scan(t(qkv), t(gates), one, t([0, T], torch.int32), slot, H, G, dk, dv)
+    whole = ops.delta_scan(t(qkv), t(gates), one, t([0, T], torch.int32), slot, H, G, dk, dv, slices)
     two = t(np.zeros((2, H, dk, dv)))
-    rows = [ops.delta_scan(t(qkv[i:i + 1]), t(gates[i:i + 1]), two, t([0, 1], torch.int32), slot, H, G, dk, dv) for i in range(T)]
+    rows = [ops.delta_scan(t(qkv[i:i + 1]), t(gates[i:i + 1]), two, t([0, 1], torch.int32), slot, H, G, dk, dv, slices) for i in range(T)]
     assert torch.equal(torch.cat([r.cpu() for r in rows]), whole.cpu()) and torch.equal(one.cpu(), two.cpu())
 
 
