@@ -195,10 +195,31 @@ experts_gather_kernel(bf16_t* __restrict__ rows, const bf16_t* __restrict__ x, c
 }
 
 // out[t, :] = sum over the token's assignments k, in order, of weights[t, k] * y[dest[t * top + k], :], in float32.
+// VEC: 16 bytes of y a thread at a time (dim a multiple of 8).
+template <bool VEC>
 __global__ void __launch_bounds__(256)
 experts_combine_kernel(float* __restrict__ out, const bf16_t* __restrict__ y, const int32_t* __restrict__ dest,
                        const float* __restrict__ weights, int top, int dim) {
     const int t = blockIdx.x;
+    if (VEC) {
+        for (int c = threadIdx.x * 8; c < dim; c += blockDim.x * 8) {
+            float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (int k = 0; k < top; ++k) {
+                const float w = weights[(size_t)t * top + k];
+                const uint4 v = *reinterpret_cast<const uint4*>(y + (size_t)dest[(size_t)t * top + k] * dim + c);
+                const uint32_t vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[2 * j] += w * __uint_as_float(vw[j] << 16);
+                    acc[2 * j + 1] += w * __uint_as_float(vw[j] & 0xFFFF0000u);
+                }
+            }
+            float4* to = reinterpret_cast<float4*>(out + (size_t)t * dim + c);
+            to[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            to[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+        }
+        return;
+    }
     for (int c = threadIdx.x; c < dim; c += blockDim.x) {
         float acc = 0.f;
         for (int k = 0; k < top; ++k)
@@ -229,7 +250,10 @@ extern "C" int ri_experts_gather(void* rows, const void* x, const int32_t* dest,
 extern "C" int ri_experts_combine(float* out, const void* y, const int32_t* dest, const float* weights, int tokens, int top,
                                   int dim, void* stream) {
     RI_REQUIRE(tokens > 0 && top >= 1 && dim >= 1, "experts_combine: %d tokens, %d a token, rows of %d", tokens, top, dim);
-    experts_combine_kernel<<<tokens, 256, 0, (hipStream_t)stream>>>(out, (const bf16_t*)y, dest, weights, top, dim);
+    if (dim % 8 == 0 && (uintptr_t)y % 16 == 0 && (uintptr_t)out % 16 == 0)
+        experts_combine_kernel<true><<<tokens, 256, 0, (hipStream_t)stream>>>(out, (const bf16_t*)y, dest, weights, top, dim);
+    else
+        experts_combine_kernel<false><<<tokens, 256, 0, (hipStream_t)stream>>>(out, (const bf16_t*)y, dest, weights, top, dim);
     RI_LAUNCH_CHECK("experts_combine");
     return 0;
 }

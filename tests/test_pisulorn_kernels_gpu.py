@@ -374,7 +374,7 @@ def test_the_experts_of_a_few_tokens(ops, T, E, top, ff, dim):
     close(got, want, BF16_OUT)
 
 
-@pytest.mark.parametrize("T, E, top, dim", [(300, 7, 3, 40), (70, 5, 1, 16), (9, 3, 3, 8), (1, 70, 4, 24), (520, 2, 1, 8)])
+@pytest.mark.parametrize("T, E, top, dim", [(300, 7, 3, 40), (70, 5, 1, 16), (9, 3, 3, 8), (1, 70, 4, 24), (520, 2, 1, 8), (5, 4, 2, 2056)])
 def test_the_assignments_sorted_by_expert(ops, T, E, top, dim):
     rng = np.random.default_rng(T)
     ids = np.stack([rng.permutation(E)[:top] for _ in range(T)]).astype(np.int32)
@@ -392,6 +392,15 @@ def test_the_assignments_sorted_by_expert(ops, T, E, top, dim):
     y = bf16_round(rng.normal(size=(T * top, dim)))
     got = ops.experts_combine(t(y, torch.bfloat16), dest, t(weights))
     close(got, (weights[:, :, None] * y[want_dest].reshape(T, top, dim)).sum(1), F32)
+
+
+def test_the_weighted_sum_of_rows_of_an_odd_size(ops):
+    rng = np.random.default_rng(2)
+    T, top, dim = 6, 3, 21
+    dest = rng.permutation(T * top).astype(np.int32)
+    y, weights = bf16_round(rng.normal(size=(T * top, dim))), rng.uniform(0.1, 1, size=(T, top))
+    got = ops.experts_combine(t(y, torch.bfloat16), t(dest, torch.int32), t(weights))
+    close(got, (weights[:, :, None] * y[dest].reshape(T, top, dim)).sum(1), F32)
 
 
 def test_an_experts_rows_activated_without_weights(ops):
