@@ -82,7 +82,9 @@ class GatedDeltaRule(Mixer):
         with profiler.section(profiler.QKV_PROJECTION):
             proj = ops.as_rows(rt.linear_packed(x, self.w_qkvg))          # [T, q | k | v | g]
             ab = rt.linear_packed(x, self.w_ab, out_dtype=torch.float32)
-        if ctx.is_decode and ops.delta_step_fits(self.dim, self.vdim):
+        # float32 and the invariant mode run one form of every kernel whatever the step looks like
+        one_form = rt.dtype == torch.float32 or rt.invariant
+        if ctx.is_decode and not one_form and ops.delta_step_fits(self.dim, self.vdim):
             # one token a sequence: convolutions, unit norms, gates, the step on the state, norm and gate are one kernel
             with profiler.section(profiler.ATTENTION):
                 y = ops.delta_step(proj, 0, self.channels, self.conv_taps, tails, ab, self.a_log, self.dt_bias, state,
@@ -94,7 +96,7 @@ class GatedDeltaRule(Mixer):
             qkv, gates = ops.delta_prepare(proj, 0, self.conv_taps, tails, ab, self.a_log, self.dt_bias, ctx.tok_seq,
                                            ctx.cu_seqlens, ctx.slots, self.heads, self.kv_heads, self.dim, self.vdim)
             o = ops.delta_scan(qkv, gates, state, ctx.cu_seqlens, ctx.slots, self.heads, self.kv_heads, self.dim,
-                               self.vdim)
+                               self.vdim, slices=4 if one_form else 0)
             y = ops.gla_norm_gate(o, proj, self.channels, self.gain, self.eps, self.heads, self.vdim)
         with profiler.section(profiler.OUT_PROJECTION):
             return rt.linear_packed(y, self.w_o, out_dtype=torch.float32, parts_ok=True)

@@ -239,6 +239,19 @@ def test_unequal_batches_one_after_another(folders, name, dtype_name):
         close_enough(got[rid][:n], alone[rid][:n].astype(np.float64), dtype_name, f"{rid}: in a batch against itself alone", bound)
 
 
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_float32_gives_the_same_bits_alone_and_in_a_batch(folders, name):
+    """float32 has one form of every kernel: three unequal requests prefilled together and decoded together, and each
+    alone with the same cut, give the same logits bit for bit."""
+    rng = np.random.default_rng(11)
+    batch = {f"{name}{i}": ([int(t) for t in rng.integers(0, CONFIGS[name]["vocab"], p + 9)], p) for i, p in enumerate(LENGTHS[name])}
+    model = loaded(folders, name, "float32")
+    together = replay(model, plans.unequal_batches([batch]))
+    for rid, (toks, p) in batch.items():
+        alone = replay(model, plans.unequal_batches([{rid: (toks, p)}]))
+        assert np.array_equal(together[rid].view(np.int32), alone[rid].view(np.int32)), f"{rid} differs from itself alone"
+
+
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_long_decoding_from_the_first_tokens(folders, name, dtype_name):
